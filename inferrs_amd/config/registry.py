@@ -19,6 +19,7 @@ from typing import Any, Dict, Optional, Type
 
 from .base import ConfigError, read_config_json
 from .buketar import BuketarConfig
+from .fisanex import FisanexConfig
 from .lofudra import LofudraConfig
 from .qwen3 import Qwen3Config
 from .spec import ModelSpec
@@ -72,3 +73,4 @@ def load_spec(model_dir: str) -> ModelSpec:
 register_architecture(Qwen3Config)
 register_architecture(BuketarConfig)
 register_architecture(LofudraConfig)
+register_architecture(FisanexConfig)

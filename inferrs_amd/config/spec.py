@@ -69,11 +69,26 @@ class AttentionSpec:
     sink: bool = False                     # the softmax's denominator holds one more term, exp(0): a key of score 0 without a value
     values_from_keys: bool = False         # no value projection: a value is the key projection's own row, taken ahead of the per-head norm and the turn by position
     names: Optional[Tuple[Tuple[str, str], ...]] = None    # (the part's tensor name, the name in the file) where they differ
+    v_head_dim: Optional[int] = None       # the width of a head's values (and of its output); None: head_dim
+    gate: bool = False                     # the joined heads are multiplied by sigmoid(W_g h) ("g_proj.weight") before the output projection
+    own_kv: bool = True                    # False: no key or value projection (nor the keys' norm): the layer's stop of the schedule reads
+                                           # another stop's cache (`ScheduleEntry.cache_of`) with its own queries, window and scale
+    reader_windows: Tuple[Optional[int], ...] = ()   # the windows of the stops that read this layer's cache: it keeps what the widest needs
     kind: str = "attention"
 
     @property
     def softmax_scale(self) -> float:
         return self.scale if self.scale is not None else self.head_dim ** -0.5
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
+
+    @property
+    def kept_window(self) -> Optional[int]:
+        """How many of the last positions the cache keeps: enough for this layer's window and for every reader's."""
+        windows = (self.window,) + tuple(self.reader_windows)
+        return None if any(w is None for w in windows) else max(windows)
 
 
 @dataclass(frozen=True)
@@ -85,6 +100,7 @@ class GatedMlpSpec:
     activation: str = "silu"
     bias: bool = False
     kind: str = "gated_mlp"
+    names: Optional[Tuple[Tuple[str, str], ...]] = None    # (the part's tensor name, the name in the file) where they differ
 
 
 @dataclass(frozen=True)
@@ -208,7 +224,11 @@ class RoutedExpertsSpec:
     """`experts` gated feed-forwards of which a token runs `top`, chosen by the router's scores (`score`:
     "sigmoid" of each logit, or "softmax" over all); weights = score * `scale`, over the chosen ones
     renormalised to 1 first with `renormalize`.  An expert: g = min(W_gate h, limit), u = clamp(W_up h, -limit,
-    limit), W_down (g * sigmoid(alpha g) * (u + 1)).  No biases."""
+    limit), W_down (g * sigmoid(alpha g) * (u + 1)).  No biases.
+    `identity`: the router has that many more outputs behind the experts'; one of them, chosen, stands for an expert
+    that hands its input on.  `correction`: a tensor "correction" [experts + identity] is added to the scores for the
+    choice only; the weights are the scores themselves.  `shared`: a `ClampedMlpSpec` that runs for every token beside
+    the chosen experts (tensors under "shared."), its output added."""
     hidden: int
     intermediate: int
     experts: int
@@ -218,7 +238,28 @@ class RoutedExpertsSpec:
     alpha: float = 1.702
     score: str = "sigmoid"
     renormalize: bool = False
+    identity: int = 0
+    correction: bool = False
+    shared: Any = None
     kind: str = "routed_experts"
+
+
+@dataclass(frozen=True)
+class ClampedMlpSpec:
+    """A gated feed-forward in the form of a routed expert, for every token: g = min(W_gate h, limit), u = clamp(W_up h,
+    -limit, limit), W_down (g * sigmoid(alpha g) * (u + 1)).  Tensors "gate", "up", "down"; no biases."""
+    hidden: int
+    intermediate: int
+    limit: float
+    alpha: float = 1.702
+    kind: str = "clamped_mlp"
+
+
+@dataclass(frozen=True)
+class PostNormSpec:
+    """How a layer's sub-layers stand around a stream that is normed after every sum (kept in 32-bit):
+    x <- norm(alpha x + part(x)), the parts reading x as it stands."""
+    alpha: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -244,7 +285,8 @@ class LayerSpec:
     feed-forward; "sandwich_norm" has a norm before and a norm behind each sub-layer around a 32-bit stream (norms in the
     order before the mixer, behind it, before the feed-forward, behind it; two norms for a layer without a feed-forward);
     "streams" is pre-norm around several residual streams (`residual`: a `StreamsSpec`) and takes a
-    layer without a feed-forward (`ffn` None, one norm).  `norms[i]` loads its weight from `norm_names[i]`."""
+    layer without a feed-forward (`ffn` None, one norm); "post_norm" norms the stream after every sum (`residual`: a
+    `PostNormSpec`; norms in the order behind the mixer, behind the feed-forward; one norm for a layer without one).  `norms[i]` loads its weight from `norm_names[i]`."""
     mixer: Any
     ffn: Any
     norms: Tuple[NormSpec, ...]
@@ -257,11 +299,14 @@ class LayerSpec:
 
 @dataclass(frozen=True)
 class EmbeddingSpec:
-    """Token ids -> rows of the stream.  kind "embedding": a gather from a [vocab, hidden] table."""
+    """Token ids -> rows of the stream.  kind "embedding": a gather from a [vocab, hidden] table, times `scale`;
+    `wide`: the rows leave in 32-bit whatever the table is stored in (for a stream that is kept so)."""
     vocab_size: int
     hidden: int
     name: str
     kind: str = "embedding"
+    scale: float = 1.0
+    wide: bool = False
 
 
 @dataclass(frozen=True)
@@ -279,12 +324,13 @@ class CappedHeadSpec:
 class HeadSpec:
     """Normed rows -> logits.  kind "lm_head": a product with a [vocab, hidden] matrix stored under
     `name`; when the file has no such tensor (or `name` is None) the embedding table serves.
-    `required`: a random model is written with a matrix of its own."""
+    `required`: a random model is written with a matrix of its own.  `scale`: a factor on the logits."""
     vocab_size: int
     hidden: int
     name: Optional[str]
     required: bool = True
     kind: str = "lm_head"
+    scale: float = 1.0
 
 
 @dataclass(frozen=True)

@@ -43,14 +43,22 @@ int ia_qk_rope_kv(void* q_out, void* k_cache, void* v_cache, const void* qkv,
                   int interleaved, int page_size, float eps, int add_one, int dtype,
                   hipStream_t stream);
 
+// The same on rows of any layout (`ld_` elements a row: queries from q_off, keys from k_off, values of width dv from v_off; k_off < 0:
+// no keys or values, the layer reads another layer's cache)
+int ia_qk_rope_kv_strided(void* q_out, void* k_cache, void* v_cache, const void* proj, const float* q_norm_w,
+                          const float* k_norm_w, const float* cos_t, const float* sin_t, const int* slots, int n,
+                          int ld_, int q_off, int k_off, int v_off, int nq, int nkv, int d, int dv, int rot,
+                          int interleaved, int page_size, float eps, int add_one, int dtype, hipStream_t stream);
+
+// d: the keys' width, dv: the values' (v_cache [pages, nkv, dv, page_size], out [n, nq, dv])
 // sink: 1 adds exp(0) to the softmax's denominator (a key of score 0 that has no value); the same in the matrix-core kernels.
 // workspace: null, or ia_attention_generic_workspace(...) floats when that is not 0 (steps of few tokens: a wave a
 // segment of keys and a merge kernel, the same bits as without); max_kv_len: an upper bound of positions + 1
 int ia_attention_generic(void* out, const void* q, const void* k_cache, const void* v_cache,
                          const int* positions, const int* token_seq, const int* block_table,
-                         int n, int max_pages, int nq, int nkv, int d, int page_size, int window,
+                         int n, int max_pages, int nq, int nkv, int d, int dv, int page_size, int window,
                          float scale, int dtype, float* workspace, int max_kv_len, int sink, hipStream_t stream);
-long long ia_attention_generic_workspace(int n, int nq, int nkv, int d, int max_kv_len);
+long long ia_attention_generic_workspace(int n, int nq, int nkv, int d, int dv, int max_kv_len);
 
 int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, int in_dtype,
                   int out_dtype, hipStream_t stream);
@@ -178,8 +186,10 @@ int ia_rglru_scan_chunked(void* out, float* state, float* work, const float* u, 
 // of one call agree).  tiled: the weights are stored as tiles of 64 features x 64 k values, zero-padded: w_gu
 // [E][2][ceil(ff / 64)][ceil(W / 64)][64][64], w_down [E][ceil(W / 64)][ceil(ff / 64)][64][64] (bfloat16, matrix cores);
 // else w_gu [E][2 ff][W], w_down [E][W][ff].
+// choice_bias: null, or [E] 32-bit values that count in the choice only (score + bias picks, the score weighs).  The plan
+// gives a pair whose choice is E or beyond (an output of the router that names no expert with weights) no place and no tile.
 int ia_route(int* sel, float* weight, const void* h, const void* router, int n, int W, int E, int top,
-             float scale, int score_fn, int renorm, int dtype, hipStream_t stream);
+             float scale, int score_fn, int renorm, const float* choice_bias, int dtype, hipStream_t stream);
 int ia_route_tiles(int pairs, int E);
 int ia_route_plan(int* order, int* tile_expert, int* tile_first, int* tile_rows, int* meta, const int* sel,
                   int pairs, int E, int tile, hipStream_t stream);
@@ -198,6 +208,23 @@ int ia_sandwich_step(float* x, const void* y1, float s1, const void* y2, float s
                      const int* rows, int n, int W, int y_dtype, int h_dtype, hipStream_t stream);
 // act over every element in place: 1 SiLU, 2 GELU in its tanh form, 3 the exact GELU
 int ia_activation(void* x, long long n, int act, int dtype, hipStream_t stream);
+
+// A 32-bit residual stream that is normed after every sum (postnorm.hip): x <- rmsnorm(alpha x + y + sum_k routed_w[k] *
+// routed[k] + y2) * w, written back in 32-bit and to h (h_dtype; null: not wanted); every addend may be null.  routed
+// [n, top, W] 32-bit with weights [n, top]; a pair whose sel (null: none) is real_experts or more stands for the stream's
+// own row.  rows: only these rows are read, the stream is left alone and h gets one row for each.
+int ia_postnorm_step(float* x, float alpha, const void* y, const void* y2, const float* routed,
+                     const float* routed_w, const int* sel, int top, int real_experts, const float* w, float eps,
+                     void* h, const int* rows, int n, int W, int y_dtype, int h_dtype, hipStream_t stream);
+// out (32-bit) = table[ids] * scale; h (null: not wanted): the same rows in the table's precision
+int ia_embed_gather_scaled(float* out, void* h, const void* table, const int* ids, int n, int hidden, int vocab,
+                           float scale, int dtype, hipStream_t stream);
+// a[row][c] *= sigmoid(g[row * g_ld + g_off + c]) in place, a [rows, cols]
+int ia_sigmoid_gate(void* a, const void* g, int rows, int cols, int g_ld, int g_off, int dtype, hipStream_t stream);
+// rows of [gate | up] -> g' * sigmoid(slope g') * (u' + 1) with g' = min(gate, limit), u' = clamp(up, -limit, limit)
+int ia_clamped_gate_mul(void* out, const void* gu, int rows, int inter, float limit, float slope, int dtype,
+                        hipStream_t stream);
+int ia_scale(float* x, long long n, float factor, hipStream_t stream);
 // Mixers with a matrix state a head (linear_state.hip).  A request's state is its row of `state` [slots][row_floats];
 // every kernel takes the offset of its part of the row.
 int ia_conv_act_step(void* out, const void* x, const void* taps, const void* bias, float* state,

@@ -56,14 +56,14 @@ __device__ __forceinline__ float ag_merge_value(float big, float a, float part, 
 // four neighbouring keys of a value's dimension are fetched with one load.  HEADS: query heads of a group (1 to 4).
 template <typename T, bool VEC, int HEADS, bool AHEAD>
 __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
-    T* __restrict__ out,                 // [n, nq, d]
+    T* __restrict__ out,                 // [n, nq, dv]
     const T* __restrict__ q,             // [n, nq, d]
     const T* __restrict__ k_cache,       // [pages, nkv, page_size, d]
-    const T* __restrict__ v_cache,       // [pages, nkv, d, page_size]  (transposed inside a page)
+    const T* __restrict__ v_cache,       // [pages, nkv, dv, page_size]  (transposed inside a page; dv: the values' width)
     const int* __restrict__ positions,   // [n]
     const int* __restrict__ token_seq,   // [n] row of block_table
     const int* __restrict__ block_table, // [seqs, max_pages]
-    int max_pages, int nq, int nkv, int d, int page_size, int window, float scale,
+    int max_pages, int nq, int nkv, int d, int dv, int page_size, int window, float scale,
     float* __restrict__ partial,         // null: a wave walks all segments; else [n, nq, segs, dpad + 2], a wave a segment
     int segs,
     int sink) {                          // 1: the softmax's denominator holds one more term, exp(0): a key of score 0 without a value
@@ -83,8 +83,9 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
     const int pos = positions[tok];
     const int* bt = block_table + (size_t)token_seq[tok] * max_pages;
     const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
-    const int chunks = (d + AG_CHUNK - 1) / AG_CHUNK;
-    const int dpad = chunks * AG_CHUNK;
+    const int chunks = (d + AG_CHUNK - 1) / AG_CHUNK;                  // of a key's dimensions
+    const int vchunks = (dv + AG_CHUNK - 1) / AG_CHUNK;                // of a value's
+    const int dpad = (chunks > vchunks ? chunks : vchunks) * AG_CHUNK;
     float* const sq = ag_rows;
     float* const so = ag_rows + HEADS * dpad;
     float* const st_ = ag_rows + 2 * HEADS * dpad;
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
         // would cost them a tenth of their speed.)
         constexpr int LOADS = AG_TILE / 4;
         static_assert(AG_TILE == AG_CHUNK, "a step of either kind is as many loads");
-        const int steps = 2 * chunks;
+        const int steps = chunks + vchunks;
         float4 held[LOADS];
         // keys: a load instruction takes four keys' rows of the chunk, 16 lanes a row, four dimensions a lane;
         // values: four dimensions, 16 lanes a dimension, four neighbouring keys a lane (four keys never straddle a page)
@@ -210,7 +211,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
                 for (int i = 0; i < LOADS; ++i) {
                     const int e = c * AG_CHUNK + 4 * i + (lane >> 4);
                     held[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (any && e < d) held[i] = ag_load4(v_cache + (((size_t)page * nkv + kvh) * d + e) * page_size + off);
+                    if (any && e < dv) held[i] = ag_load4(v_cache + (((size_t)page * nkv + kvh) * dv + e) * page_size + off);
                 }
             }
         };
@@ -296,7 +297,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
             scores(c);
         }
         softmax(valid);
-        for (int c = 0; c < chunks; ++c) {
+        for (int c = 0; c < vchunks; ++c) {
             __syncthreads();                                          // the stage is free, the probabilities are there
             if constexpr (VEC) {
                 // a load instruction takes four dimensions: 16 lanes a dimension, four neighbouring keys a lane
@@ -313,8 +314,8 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
                 for (int i = 0; i < AG_CHUNK / 4; ++i) {
                     const int e = c * AG_CHUNK + 4 * i + (lane >> 4);
                     v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (any && e < d) {
-                        v[i] = ag_load4(v_cache + (((size_t)page * nkv + kvh) * d + e) * page_size + off);
+                    if (any && e < dv) {
+                        v[i] = ag_load4(v_cache + (((size_t)page * nkv + kvh) * dv + e) * page_size + off);
                         v[i].x = (key >= lo && key <= pos) ? v[i].x : 0.f;
                         v[i].y = (key + 1 >= lo && key + 1 <= pos) ? v[i].y : 0.f;
                         v[i].z = (key + 2 >= lo && key + 2 <= pos) ? v[i].z : 0.f;
@@ -329,7 +330,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
                 for (int r = 0; r < AG_CHUNK; ++r) {
                     const int e = c * AG_CHUNK + r;
                     stage[r * AG_PITCH + lane] =
-                        (valid && e < d) ? ld(v_cache + (((size_t)my_page * nkv + kvh) * d + e) * page_size + off) : 0.f;
+                        (valid && e < dv) ? ld(v_cache + (((size_t)my_page * nkv + kvh) * dv + e) * page_size + off) : 0.f;
                 }
             }
             __syncthreads();
@@ -361,9 +362,9 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
 #pragma unroll
     for (int h = 0; h < HEADS; ++h) {
         if (h >= heads) break;
-        T* orow = out + ((size_t)tok * nq + h0 + h) * d;
+        T* orow = out + ((size_t)tok * nq + h0 + h) * dv;
         const float inv = 1.0f / (sink ? big_l[h] + expf(-big_m[h]) : big_l[h]);
-        for (int e = lane; e < d; e += IA_WAVE) st(orow + e, st_[h * dpad + e] * inv);
+        for (int e = lane; e < dv; e += IA_WAVE) st(orow + e, st_[h * dpad + e] * inv);
     }
 }
 
@@ -405,24 +406,25 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_merge_kernel(
 
 // Floats of the workspace that steps of few tokens need (0: the step has tokens enough for a wave each to walk
 // all its segments).  `max_kv_len`: an upper bound of the positions + 1.
-extern "C" long long ia_attention_generic_workspace(int n, int nq, int nkv, int d, int max_kv_len) {
-    if (n <= 0 || nq <= 0 || nkv <= 0 || d <= 0 || max_kv_len <= AG_SEGMENT) return 0;
+extern "C" long long ia_attention_generic_workspace(int n, int nq, int nkv, int d, int dv, int max_kv_len) {
+    if (n <= 0 || nq <= 0 || nkv <= 0 || d <= 0 || dv <= 0 || max_kv_len <= AG_SEGMENT) return 0;
     const int g = nq / nkv;
     const int per_group = g < AG_HEADS ? g : AG_HEADS;
     const long long units = (long long)n * nkv * ((g + per_group - 1) / per_group);
     if (units >= 2048) return 0;
     const int segs = (max_kv_len + AG_SEGMENT - 1) / AG_SEGMENT;
-    const int dpad = (d + AG_CHUNK - 1) / AG_CHUNK * AG_CHUNK;
+    const int dpad = ((d > dv ? d : dv) + AG_CHUNK - 1) / AG_CHUNK * AG_CHUNK;
     return (long long)n * nq * segs * (dpad + 2);
 }
 
 extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cache, const void* v_cache,
                                     const int* positions, const int* token_seq, const int* block_table,
-                                    int n, int max_pages, int nq, int nkv, int d, int page_size,
+                                    int n, int max_pages, int nq, int nkv, int d, int dv, int page_size,
                                     int window, float scale, int dtype, float* workspace, int max_kv_len,
                                     int sink, hipStream_t stream) {
     IA_CHECK(n >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention: bad head counts nq=%d nkv=%d (n=%d)", nq, nkv, n);
     IA_CHECK(d > 0 && d <= AG_MAX_HEAD_DIM, "attention: head_dim %d is outside 1..%d", d, AG_MAX_HEAD_DIM);
+    IA_CHECK(dv > 0 && dv <= AG_MAX_HEAD_DIM, "attention: the values' width %d is outside 1..%d", dv, AG_MAX_HEAD_DIM);
     IA_CHECK(page_size > 0 && max_pages > 0, "attention: bad page geometry page_size=%d max_pages=%d", page_size, max_pages);
     IA_CHECK(window >= 0, "attention: window %d must be >= 0 (0 = all keys)", window);
     if (n == 0) return 0;
@@ -432,18 +434,18 @@ extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cach
     IA_CHECK((long long)n * nkv * groups < 2147483647LL, "attention: %d tokens x %d heads exceed the grid", n, nq);
     // a wave a segment when the workspace is given (ia_attention_generic_workspace says when it is needed)
     const int segs = workspace != nullptr ? (max_kv_len + AG_SEGMENT - 1) / AG_SEGMENT : 1;
-    IA_CHECK(workspace == nullptr || (max_kv_len > 0 && ia_attention_generic_workspace(n, nq, nkv, d, max_kv_len) > 0),
+    IA_CHECK(workspace == nullptr || (max_kv_len > 0 && ia_attention_generic_workspace(n, nq, nkv, d, dv, max_kv_len) > 0),
              "attention: a workspace goes with max_kv_len and a step of few tokens");
     IA_CHECK((long long)n * nkv * groups * segs < 2147483647LL, "attention: %d tokens x %d heads exceed the grid", n, nq);
     const unsigned grid = (unsigned)n * (unsigned)nkv * (unsigned)groups * (unsigned)segs;
-    const int dpad = (d + AG_CHUNK - 1) / AG_CHUNK * AG_CHUNK;
-    const size_t rows_bytes = (size_t)3 * per_group * ((d + AG_CHUNK - 1) / AG_CHUNK * AG_CHUNK) * sizeof(float);
+    const int dpad = ((d > dv ? d : dv) + AG_CHUNK - 1) / AG_CHUNK * AG_CHUNK;
+    const size_t rows_bytes = (size_t)3 * per_group * dpad * sizeof(float);
     const size_t elem = dtype == IA_F32 ? 4 : 2;
     // loads of four elements: rows of the caches start at multiples of four elements, on aligned arrays
-    const bool vec = d % 4 == 0 && page_size % 4 == 0 &&
+    const bool vec = d % 4 == 0 && dv % 4 == 0 && page_size % 4 == 0 &&
                      (((uintptr_t)k_cache | (uintptr_t)v_cache) % (4 * elem)) == 0;
 #define AG_ARGS(T) (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache, positions, token_seq, block_table, max_pages, nq, nkv, \
-        d, page_size, window, scale, workspace, segs, sink
+        d, dv, page_size, window, scale, workspace, segs, sink
     // (a wave a segment, steps of few tokens: the operands are asked for a step ahead)
 #define AG_LAUNCH(T, V, H) do { \
         if (V && workspace != nullptr) attn_generic_kernel<T, V, H, true><<<grid, IA_WAVE, rows_bytes, stream>>>(AG_ARGS(T)); \
@@ -460,9 +462,9 @@ extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cach
     IA_LAUNCH_CHECK("attention_generic");
     if (workspace != nullptr) {
         if (dtype == IA_F32)
-            attn_generic_merge_kernel<float><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((float*)out, workspace, positions, nq, d, dpad, window, segs, sink);
+            attn_generic_merge_kernel<float><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((float*)out, workspace, positions, nq, dv, dpad, window, segs, sink);
         else
-            attn_generic_merge_kernel<bf16_t><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((bf16_t*)out, workspace, positions, nq, d, dpad, window, segs, sink);
+            attn_generic_merge_kernel<bf16_t><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((bf16_t*)out, workspace, positions, nq, dv, dpad, window, segs, sink);
         IA_LAUNCH_CHECK("attention_generic_merge");
     }
     return 0;

@@ -45,7 +45,7 @@ template <typename T, bool VEC>
 __global__ __launch_bounds__(64 * IA_ROUTE_WAVES) void route_kernel(int* __restrict__ sel, float* __restrict__ weight,
                                                                     const T* __restrict__ h, const T* __restrict__ wr, int n,
                                                                     int W, int E, int top, float scale, int score_fn,
-                                                                    int renorm) {
+                                                                    int renorm, const float* __restrict__ choice_bias) {
     __shared__ float logits[IA_MAX_EXPERTS];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const T* row = h + (long long)t * W;
@@ -104,6 +104,35 @@ __global__ __launch_bounds__(64 * IA_ROUTE_WAVES) void route_kernel(int* __restr
     }
     float total = 0.f, mine = 0.f;
     int mine_e = 0;
+    if (choice_bias != nullptr) {
+        // The choice goes by score + bias, the weights by the score alone: the scores are formed first, and the picking
+        // walks the biased ones (of equal ones the lower index).
+        float sc[IA_MAX_EXPERTS / IA_WAVE], key[IA_MAX_EXPERTS / IA_WAVE];
+#pragma unroll
+        for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) {
+            const int e = q * IA_WAVE + lane;
+            sc[q] = e < E ? (score_fn == IA_SCORE_SOFTMAX ? expf(z[q] - zmax) / denom : 1.0f / (1.0f + expf(-z[q]))) : 0.f;
+            key[q] = e < E ? sc[q] + choice_bias[e] : -INFINITY;
+        }
+        for (int k = 0; k < top; ++k) {
+            float best = -INFINITY, best_s = 0.f;
+            int best_e = 0x7fffffff;
+#pragma unroll
+            for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q)
+                if (key[q] > best) { best = key[q]; best_e = q * IA_WAVE + lane; best_s = sc[q]; }
+#pragma unroll
+            for (int o = IA_WAVE / 2; o > 0; o >>= 1) {
+                const float ob = __shfl_xor(best, o, IA_WAVE), os = __shfl_xor(best_s, o, IA_WAVE);
+                const int oe = __shfl_xor(best_e, o, IA_WAVE);
+                if (ob > best || (ob == best && oe < best_e)) { best = ob; best_e = oe; best_s = os; }
+            }
+#pragma unroll
+            for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q)
+                if (best_e == q * IA_WAVE + lane) key[q] = -INFINITY;
+            total += best_s;
+            if (lane == k) { mine = best_s; mine_e = best_e; }
+        }
+    } else
     for (int k = 0; k < top; ++k) {
         // every lane's best, then the wave's: the largest logit, of equal ones the lower index
         float best = -INFINITY;
@@ -138,7 +167,9 @@ __global__ __launch_bounds__(1024) void route_plan_kernel(int* __restrict__ orde
     __shared__ int count[IA_MAX_EXPERTS], first[IA_MAX_EXPERTS], tile0[IA_MAX_EXPERTS], cursor[IA_MAX_EXPERTS];
     for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = cursor[e] = 0;
     __syncthreads();
-    for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&count[sel[p]], 1);
+    // (a choice of E or beyond names no expert with weights: such a pair gets no place and no tile)
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x)
+        if (sel[p] < E) atomicAdd(&count[sel[p]], 1);
     __syncthreads();
     if (threadIdx.x == 0) {
         int at = 0, tiles = 0;
@@ -161,7 +192,7 @@ __global__ __launch_bounds__(1024) void route_plan_kernel(int* __restrict__ orde
     }
     for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
         const int e = sel[p];
-        order[first[e] + atomicAdd(&cursor[e], 1)] = p;
+        if (e < E) order[first[e] + atomicAdd(&cursor[e], 1)] = p;
     }
 }
 
@@ -293,14 +324,15 @@ __global__ __launch_bounds__(256) void experts_down_mfma_kernel(float* __restric
     });
 }
 
+// choice_bias: null, or [E] 32-bit values added to the scores for the choice only (the weights are the scores themselves)
 extern "C" int ia_route(int* sel, float* weight, const void* h, const void* router, int n, int W, int E, int top,
-                        float scale, int score_fn, int renorm, int dtype, hipStream_t stream) {
+                        float scale, int score_fn, int renorm, const float* choice_bias, int dtype, hipStream_t stream) {
     IA_CHECK(n >= 0 && W > 0 && E >= 1 && E <= IA_MAX_EXPERTS && top >= 1 && top <= E && top <= IA_MAX_TOP,
              "route: n=%d width=%d experts=%d (up to %d) top=%d (up to %d)", n, W, E, IA_MAX_EXPERTS, top, IA_MAX_TOP);
     IA_CHECK(score_fn == IA_SCORE_SIGMOID || score_fn == IA_SCORE_SOFTMAX, "route: unknown score function %d", score_fn);
     if (n == 0) return 0;
     const bool vec = W % 8 == 0 && tile_mfma_aligned(h) && tile_mfma_aligned(router);
-#define IA_ROUTE(T, V) route_kernel<T, V><<<n, 64 * IA_ROUTE_WAVES, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm)
+#define IA_ROUTE(T, V) route_kernel<T, V><<<n, 64 * IA_ROUTE_WAVES, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm, choice_bias)
     if (dtype == IA_F32) { if (vec) IA_ROUTE(float, true); else IA_ROUTE(float, false); }
     else { if (vec) IA_ROUTE(bf16_t, true); else IA_ROUTE(bf16_t, false); }
 #undef IA_ROUTE

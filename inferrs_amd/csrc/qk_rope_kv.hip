@@ -86,6 +86,113 @@ __global__ __launch_bounds__(QK_WAVES * IA_WAVE) void qk_rope_kv_kernel(
     for (int j = rot + lane; j < d; j += IA_WAVE) st(dst + j, row[j]);
 }
 
+// The same work on rows of any layout: the projections' output holds a token's query heads from `q_off`, its key heads
+// from `k_off` and its value heads (each `dv` wide, which need not be the keys' width) from `v_off`, `ld` elements a
+// row; whatever else the row holds (a gate, say) is left alone.  `k_off` < 0 or no slots: the layer writes no cache
+// (it reads another layer's), and only the queries are formed.  One wave per (token, head).
+template <typename T>
+__global__ __launch_bounds__(QK_WAVES * IA_WAVE) void qk_rope_kv_strided_kernel(
+    T* __restrict__ q_out,              // [n, nq, d]
+    T* __restrict__ k_cache,            // [pages, nkv, page_size, d] or null
+    T* __restrict__ v_cache,            // [pages, nkv, dv, page_size] or null
+    const T* __restrict__ proj,         // [n, ld]
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, const int* __restrict__ slots,
+    int n, int ld_, int q_off, int k_off, int v_off, int nq, int nkv, int d, int dv, int rot, int interleaved,
+    int page_size, float eps, int add_one) {
+    __shared__ float buf[QK_WAVES][QK_MAX_HEAD_DIM];
+    const int lane = threadIdx.x & (IA_WAVE - 1);
+    const int wave = threadIdx.x / IA_WAVE;
+    const int heads = slots ? nq + 2 * nkv : nq;
+    const long long unit = (long long)blockIdx.x * QK_WAVES + wave;
+    const bool active = unit < (long long)n * heads;
+    const int tok = active ? (int)(unit / heads) : 0;
+    const int hh = active ? (int)(unit % heads) : 0;
+    const int kind = hh < nq ? 0 : (hh < nq + nkv ? 1 : 2);
+    const int width = kind == 2 ? dv : d;
+    const T* src = proj + (size_t)tok * ld_ +
+                   (kind == 0 ? q_off + hh * d : kind == 1 ? k_off + (hh - nq) * d : v_off + (hh - nq - nkv) * dv);
+    float* row = buf[wave];
+
+    float ss = 0.f;
+    if (active) {
+        for (int j = lane; j < width; j += IA_WAVE) {
+            const float v = ld(src + j);
+            row[j] = v;
+            ss += v * v;
+        }
+    }
+    const float* nw = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
+    if (nw != nullptr) {
+        ss = wave_sum(ss);
+        const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+        if (active)
+            for (int j = lane; j < d; j += IA_WAVE) row[j] = scale * row[j] * (add_one ? 1.0f + nw[j] : nw[j]);
+    }
+    __syncthreads();
+    if (!active) return;
+
+    T* dst;
+    if (kind == 0) {
+        dst = q_out + ((size_t)tok * nq + hh) * d;
+    } else {
+        const int slot = slots[tok];
+        const int page = slot / page_size, off = slot - page * page_size;
+        if (kind == 2) {
+            // values are kept transposed inside a page: [dim][slot]
+            T* vt = v_cache + ((size_t)page * nkv + (hh - nq - nkv)) * dv * page_size + off;
+            for (int j = lane; j < dv; j += IA_WAVE) st(vt + (size_t)j * page_size, row[j]);
+            return;
+        }
+        dst = k_cache + (((size_t)page * nkv + (hh - nq)) * page_size + off) * d;
+    }
+    if (cos_t == nullptr) {
+        for (int j = lane; j < d; j += IA_WAVE) st(dst + j, row[j]);
+        return;
+    }
+    const int half = rot / 2;
+    for (int i = lane; i < half; i += IA_WAVE) {
+        const float c = cos_t[(size_t)tok * half + i], s = sin_t[(size_t)tok * half + i];
+        const int ia = interleaved ? 2 * i : i;
+        const int ib = interleaved ? 2 * i + 1 : i + half;
+        const float a = row[ia], b = row[ib];
+        st(dst + ia, a * c - b * s);
+        st(dst + ib, a * s + b * c);
+    }
+    for (int j = rot + lane; j < d; j += IA_WAVE) st(dst + j, row[j]);
+}
+
+extern "C" int ia_qk_rope_kv_strided(void* q_out, void* k_cache, void* v_cache, const void* proj, const float* q_norm_w,
+                                     const float* k_norm_w, const float* cos_t, const float* sin_t, const int* slots, int n,
+                                     int ld_, int q_off, int k_off, int v_off, int nq, int nkv, int d, int dv, int rot,
+                                     int interleaved, int page_size, float eps, int add_one, int dtype, hipStream_t stream) {
+    IA_CHECK(n >= 0 && nq > 0 && nkv > 0, "qk_rope_kv_strided: bad sizes n=%d nq=%d nkv=%d", n, nq, nkv);
+    IA_CHECK(d > 0 && d <= QK_MAX_HEAD_DIM && dv > 0 && dv <= QK_MAX_HEAD_DIM,
+             "qk_rope_kv_strided: head sizes %d / %d are outside 1..%d", d, dv, QK_MAX_HEAD_DIM);
+    IA_CHECK(rot >= 0 && rot <= d && rot % 2 == 0, "qk_rope_kv_strided: rot_dim %d must be even and <= head_dim %d", rot, d);
+    IA_CHECK((cos_t == nullptr) == (sin_t == nullptr), "qk_rope_kv_strided: cos and sin tables must come together");
+    IA_CHECK(cos_t == nullptr || rot > 0, "qk_rope_kv_strided: a rotary table needs rot_dim > 0");
+    IA_CHECK(q_off >= 0 && q_off + nq * d <= ld_, "qk_rope_kv_strided: the queries at %d do not fit rows of %d", q_off, ld_);
+    if (k_off < 0) slots = nullptr;
+    IA_CHECK(slots == nullptr || (k_cache && v_cache && page_size > 0 && v_off >= 0 && k_off + nkv * d <= ld_ && v_off + nkv * dv <= ld_),
+             "qk_rope_kv_strided: keys at %d and values at %d need a cache and room in rows of %d", k_off, v_off, ld_);
+    if (n == 0) return 0;
+    const long long units = (long long)n * (slots ? nq + 2 * nkv : nq);
+    const unsigned grid = (unsigned)((units + QK_WAVES - 1) / QK_WAVES);
+    if (dtype == IA_F32)
+        qk_rope_kv_strided_kernel<float><<<grid, QK_WAVES * IA_WAVE, 0, stream>>>(
+            (float*)q_out, (float*)k_cache, (float*)v_cache, (const float*)proj, q_norm_w, k_norm_w, cos_t, sin_t, slots, n,
+            ld_, q_off, k_off, v_off, nq, nkv, d, dv, rot, interleaved, page_size, eps, add_one);
+    else if (dtype == IA_BF16)
+        qk_rope_kv_strided_kernel<bf16_t><<<grid, QK_WAVES * IA_WAVE, 0, stream>>>(
+            (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, (const bf16_t*)proj, q_norm_w, k_norm_w, cos_t, sin_t, slots,
+            n, ld_, q_off, k_off, v_off, nq, nkv, d, dv, rot, interleaved, page_size, eps, add_one);
+    else
+        IA_CHECK(false, "qk_rope_kv_strided: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("qk_rope_kv_strided");
+    return 0;
+}
+
 #define QKV_THREADS 256
 #define QKV_GROUP 8
 

@@ -344,24 +344,64 @@ def qk_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int, *,
     return q_out
 
 
+def qk_rope_kv_strided(proj: torch.Tensor, nq: int, nkv: int, d: int, dv: int, *, q_off: int, k_off: Optional[int],
+                       v_off: Optional[int], q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
+                       add_one: bool, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rot: int, interleaved: bool,
+                       k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+                       page_size: int) -> torch.Tensor:
+    """`qk_rope_kv` on rows of any layout: a row of `proj` holds the query heads from `q_off`, the key heads from `k_off`
+    and the value heads (`dv` wide each) from `v_off`, and whatever else beside them.  `k_off` None: the rows hold no keys
+    or values (a layer that reads another layer's cache).  Returns q [n, nq, d]."""
+    _dev(proj, q_norm_w, k_norm_w, cos, sin, k_cache, v_cache, slots)
+    _f32(q_norm_w, "q_norm weight"); _f32(k_norm_w, "k_norm weight"); _f32(cos, "cos"); _f32(sin, "sin")
+    if proj.dim() != 2 or proj.stride(1) != 1:
+        raise KernelError(f"qk_rope_kv_strided: the projections are 2-D rows, got {tuple(proj.shape)}")
+    n, ld_ = proj.shape[0], proj.stride(0)
+    for w, name in ((q_norm_w, "q_norm"), (k_norm_w, "k_norm")):
+        if w is not None and w.numel() != d:
+            raise KernelError(f"qk_rope_kv_strided: {name} weight has {w.numel()} entries, head_dim is {d}")
+    if cos is not None and (sin is None or cos.shape != (n, rot // 2) or sin.shape != cos.shape):
+        raise KernelError(f"qk_rope_kv_strided: rotary tables must be [{n}, {rot // 2}]")
+    if q_off < 0 or q_off + nq * d > proj.shape[1]:
+        raise KernelError(f"qk_rope_kv_strided: {nq} query heads of {d} at {q_off} do not fit rows of {proj.shape[1]}")
+    if k_off is None:
+        slots = None
+    if slots is not None:
+        _i32(slots, "slots")
+        if k_cache is None or v_cache is None or v_off is None or slots.numel() != n:
+            raise KernelError("qk_rope_kv_strided: slots need a cache, the values' place and one entry a token")
+        if k_off < 0 or v_off < 0 or k_off + nkv * d > proj.shape[1] or v_off + nkv * dv > proj.shape[1]:
+            raise KernelError(f"qk_rope_kv_strided: keys at {k_off} / values at {v_off} do not fit rows of {proj.shape[1]}")
+        _check_cache(k_cache, v_cache, nkv, page_size, d, proj.dtype, "qk_rope_kv_strided", dv)
+    q_out = torch.empty((n, nq, d), dtype=proj.dtype, device=proj.device)
+    _check(library().ia_qk_rope_kv_strided(
+        _p(q_out), _p(k_cache if slots is not None else None), _p(v_cache if slots is not None else None), _p(proj),
+        _p(q_norm_w), _p(k_norm_w), _p(cos), _p(sin), _p(slots), n, ld_, q_off, -1 if k_off is None else k_off,
+        -1 if v_off is None else v_off, nq, nkv, d, dv, rot, int(interleaved), page_size, ctypes.c_float(eps), int(add_one),
+        _dt(proj), _stream()))
+    return q_out
+
+
 # ---- attention --------------------------------------------------------------------------------
 
 def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, page_size: int, d: int,
-                 dtype: torch.dtype, who: str) -> None:
-    """Keys [pages, nkv, page_size, d]; values transposed inside a page, [pages, nkv, d, page_size]."""
+                 dtype: torch.dtype, who: str, dv: Optional[int] = None) -> None:
+    """Keys [pages, nkv, page_size, d]; values transposed inside a page, [pages, nkv, dv, page_size] (dv None: d)."""
+    dv = d if dv is None else dv
     if (k_cache.dtype != dtype or v_cache.dtype != dtype or k_cache.dim() != 4 or v_cache.dim() != 4
-            or tuple(k_cache.shape[1:]) != (nkv, page_size, d) or tuple(v_cache.shape[1:]) != (nkv, d, page_size)
+            or tuple(k_cache.shape[1:]) != (nkv, page_size, d) or tuple(v_cache.shape[1:]) != (nkv, dv, page_size)
             or k_cache.shape[0] != v_cache.shape[0]):
         raise KernelError(f"{who}: cache has shapes {tuple(k_cache.shape)} {k_cache.dtype} and "
                           f"{tuple(v_cache.shape)} {v_cache.dtype}, expected [pages, {nkv}, {page_size}, {d}] "
-                          f"and [pages, {nkv}, {d}, {page_size}] {dtype}")
+                          f"and [pages, {nkv}, {dv}, {page_size}] {dtype}")
 
 
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
                       *, window: Optional[int], scale: float, max_kv_len: Optional[int] = None,
                       split: Optional[bool] = None, sink: bool = False) -> torch.Tensor:
-    """q [n, nq, d] against the paged cache; token i sees the keys at positions <= positions[i]
+    """q [n, nq, d] against the paged cache (values may have a width of their own: v_cache [pages, nkv, dv, page_size],
+    the result is [n, nq, dv]); token i sees the keys at positions <= positions[i]
     (and > positions[i] - window) of row token_seq[i] of the table.  Any head size up to 512, any
     page size, 32-bit or bfloat16 storage, all arithmetic in 32-bit.  `max_kv_len`: an upper bound of
     positions + 1 (default: what the table can hold).  Steps of few tokens run a wave a segment of 512 keys
@@ -371,20 +411,21 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _i32(positions, "positions"); _i32(token_seq, "token_seq"); _i32(block_table, "block_table")
     n, nq, d = q.shape
     nkv, page_size = k_cache.shape[1], k_cache.shape[2]
-    _check_cache(k_cache, v_cache, nkv, page_size, d, q.dtype, "attention")
+    dv = v_cache.shape[2] if v_cache.dim() == 4 else d
+    _check_cache(k_cache, v_cache, nkv, page_size, d, q.dtype, "attention", dv)
     if positions.numel() != n or token_seq.numel() != n or block_table.dim() != 2:
         raise KernelError("attention: positions, token_seq and block_table do not fit the batch")
     capacity = block_table.shape[1] * page_size
     max_kv_len = capacity if max_kv_len is None else min(int(max_kv_len), capacity)
-    out = torch.empty_like(q)
+    out = torch.empty((n, nq, dv), dtype=q.dtype, device=q.device)
     lib = library()
-    ws_floats = lib.ia_attention_generic_workspace(n, nq, nkv, d, max_kv_len) if split is not False else 0
+    ws_floats = lib.ia_attention_generic_workspace(n, nq, nkv, d, dv, max_kv_len) if split is not False else 0
     if split and not ws_floats:
         raise KernelError("attention: a step of this many tokens, or of so few keys, is not split")
     ws = torch.empty((ws_floats,), dtype=torch.float32, device=q.device) if ws_floats else None
     _check(lib.ia_attention_generic(
         _p(out), _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_seq), _p(block_table), n,
-        block_table.shape[1], nq, nkv, d, page_size, int(window or 0), ctypes.c_float(scale), _dt(q),
+        block_table.shape[1], nq, nkv, d, dv, page_size, int(window or 0), ctypes.c_float(scale), _dt(q),
         _p(ws), max_kv_len, int(bool(sink)), _stream()))
     return out
 
@@ -393,8 +434,10 @@ ATTN_TARGET_WAVES = 2048       # waves wanted in flight before the keys stop bei
 ATTN_MIN_CHUNK = 64            # fewest keys a split is worth
 
 
-def attention_mfma_fits(dtype: torch.dtype, d: int, page_size: int) -> bool:
-    return dtype == torch.bfloat16 and d in _build.ATTN_HEAD_DIMS and page_size % 16 == 0
+def attention_mfma_fits(dtype: torch.dtype, d: int, page_size: int, dv: Optional[int] = None) -> bool:
+    """`dv`: the values' width where it is not the keys'."""
+    return (dtype == torch.bfloat16 and d in _build.ATTN_HEAD_DIMS and page_size % 16 == 0
+            and (dv is None or dv == d))
 
 
 ATTN_TILE_COLS = 128           # head size 128, prompt portions: columns a block of four waves
@@ -1184,7 +1227,8 @@ def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
 
 
 # ---- several residual streams, latent attention, gated recurrence, routed experts -----------------
-from .mix import (conv_step, experts_forward, head_product, latent_prep, rglru_scan, route, softcap,   # noqa: E402
+from .mix import (clamped_gate_mul, conv_step, embed_gather_scaled, experts_forward, head_product,    # noqa: E402
+                  latent_prep, postnorm_step, rglru_scan, route, scale_inplace, sigmoid_gate, softcap,
                   streams_open, streams_step)
 from .state import (activation, conv_act_step, exp_gates, group_norm_gate, linear_scan, sandwich_step,   # noqa: E402
                     step_gates)

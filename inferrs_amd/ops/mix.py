@@ -205,11 +205,14 @@ def rglru_scan(u: torch.Tensor, z: torch.Tensor, proj: torch.Tensor, *, branch_o
 # ---- routed experts -----------------------------------------------------------------------------
 
 def route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, score: str = "sigmoid",
-          renormalize: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+          renormalize: bool = False, choice_bias: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Router logits in 32-bit (router [E, width] in the precision of h; every logit is a sum of 32-bit
     multiply-adds in an order that the width alone decides), the `top` experts by score for every row:
-    (experts int32 [n, top] best first, weights float32 [n, top] = score * scale)."""
-    _dev(h, router)
+    (experts int32 [n, top] best first, weights float32 [n, top] = score * scale).  `choice_bias` [E] (32-bit):
+    the choice goes by score + bias, the weights stay the scores."""
+    _dev(h, router, choice_bias); _f32(choice_bias, "choice_bias")
+    if choice_bias is not None and choice_bias.numel() != router.shape[0]:
+        raise KernelError(f"route: {choice_bias.numel()} biases for {router.shape[0]} outputs of the router")
     n, W = h.shape
     E = router.shape[0]
     if (router.shape[1] != W or router.dtype != h.dtype or not (1 <= top <= min(E, MAX_TOP)) or E > MAX_EXPERTS
@@ -219,7 +222,7 @@ def route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, score: 
     sel = torch.empty((n, top), dtype=torch.int32, device=h.device)
     weight = torch.empty((n, top), dtype=torch.float32, device=h.device)
     _check(library().ia_route(_p(sel), _p(weight), _p(h), _p(router), n, W, E, top, ctypes.c_float(scale),
-                              SCORE_FUNCTIONS[score], int(renormalize), _dt(h), _stream()))
+                              SCORE_FUNCTIONS[score], int(renormalize), _p(choice_bias), _dt(h), _stream()))
     return sel, weight
 
 
@@ -243,7 +246,8 @@ def experts_forward(h: torch.Tensor, sel: torch.Tensor, w_gate_up: torch.Tensor,
     """The chosen experts of every row: w_gate_up [E, 2 ff, width] (gate rows, then up rows), w_down [E, width, ff],
     or both as tiles (`tile_weights` of [E, 2, ff, width] and of [E, width, ff]; then `ff` is given);
     act = g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).  Returns one
-    32-bit output row a (row, k) pair, [n, top, width]; nothing is added up here."""
+    32-bit output row a (row, k) pair, [n, top, width]; nothing is added up here.  A choice of E or beyond names no
+    expert with weights: its row is left unwritten (whoever adds the rows up knows what stands for it)."""
     _dev(h, sel, w_gate_up, w_down); _i32(sel, "sel")
     n, W = h.shape
     top = sel.shape[1]
@@ -280,3 +284,90 @@ def experts_forward(h: torch.Tensor, sel: torch.Tensor, w_gate_up: torch.Tensor,
     _check(lib.ia_experts_down(_p(y), _p(act), _p(w_down), _p(order), _p(t_exp), _p(t_first), _p(t_rows), _p(meta), pairs,
                                E, W, ff, tile, int(tiled), _dt(h), _stream()))
     return y
+
+
+# ---- a stream that is normed after every sum ------------------------------------------------------------------------
+
+def postnorm_step(x: torch.Tensor, *, alpha: float = 1.0, y: Optional[torch.Tensor] = None, y2: Optional[torch.Tensor] = None,
+                  routed: Optional[torch.Tensor] = None, routed_weights: Optional[torch.Tensor] = None,
+                  sel: Optional[torch.Tensor] = None, real_experts: int = 0, weight: torch.Tensor, eps: float,
+                  h_dtype: Optional[torch.dtype] = None, rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """What stands behind a sub-layer around a 32-bit stream x [n, width] that is normed after every sum (changed in place):
+
+        x <- rmsnorm(alpha x + y + sum_k routed_weights[:, k] * routed[:, k] + y2) * weight
+
+    and, with `h_dtype`, the new rows once more in that precision.  Every addend may be absent.  `routed` [n, top, width]
+    (32-bit): with `sel` [n, top], a pair whose entry is `real_experts` or more stands for the stream's own row (an expert
+    that hands its input on).  `rows` (int32): only these rows are read, the stream is left as it is and the result has one
+    row for each of them."""
+    _dev(x, y, y2, routed, routed_weights, sel, weight, rows)
+    _f32(x, "the stream"); _f32(routed, "routed rows"); _f32(routed_weights, "routed weights"); _f32(weight, "norm weight")
+    n, W = x.shape
+    given = [t for t in (y, y2) if t is not None]
+    for t in given:
+        if tuple(t.shape) != (n, W) or t.dtype != given[0].dtype:
+            raise KernelError(f"postnorm_step: an output {tuple(t.shape)} {t.dtype} does not fit the stream [{n}, {W}]")
+    top = 0
+    if routed is not None:
+        top = routed.shape[1]
+        if (routed.dim() != 3 or tuple(routed.shape) != (n, top, W) or routed_weights is None
+                or tuple(routed_weights.shape) != (n, top) or top > MAX_TOP):
+            raise KernelError(f"postnorm_step: routed rows {tuple(routed.shape)} and their weights do not fit [{n}, top <= {MAX_TOP}, {W}]")
+        if sel is not None:
+            _i32(sel, "sel")
+            if tuple(sel.shape) != (n, top):
+                raise KernelError(f"postnorm_step: choices {tuple(sel.shape)} do not fit [{n}, {top}]")
+    if weight.numel() != W:
+        raise KernelError(f"postnorm_step: the norm weight has {weight.numel()} entries, the stream is {W} wide")
+    count = n
+    if rows is not None:
+        _i32(rows, "rows")
+        count = rows.numel()
+        if h_dtype is None or given or routed is not None:
+            raise KernelError("postnorm_step: a row list goes with an output and nothing to add")
+    h = torch.empty((count, W), dtype=h_dtype, device=x.device) if h_dtype is not None else None
+    _check(library().ia_postnorm_step(
+        _p(x), ctypes.c_float(alpha), _p(y), _p(y2), _p(routed), _p(routed_weights), _p(sel), top, int(real_experts),
+        _p(weight), ctypes.c_float(eps), _p(h), _p(rows), count, W, _dt(given[0]) if given else 0,
+        _DT[h_dtype] if h_dtype is not None else 0, _stream()))
+    return h
+
+
+def embed_gather_scaled(table: torch.Tensor, ids: torch.Tensor, scale: float, rounded: bool = False):
+    """table[ids] * scale as 32-bit rows; `rounded`: (rows, the same rows in the table's precision)."""
+    _dev(table, ids); _i32(ids, "token ids")
+    n, (vocab, hidden) = ids.numel(), table.shape
+    out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
+    lo = torch.empty((n, hidden), dtype=table.dtype, device=table.device) if rounded else None
+    _check(library().ia_embed_gather_scaled(_p(out), _p(lo), _p(table), _p(ids), n, hidden, vocab, ctypes.c_float(scale),
+                                            _dt(table), _stream()))
+    return (out, lo) if rounded else out
+
+
+def sigmoid_gate(a: torch.Tensor, g: torch.Tensor, g_off: int = 0) -> torch.Tensor:
+    """a[:, c] *= sigmoid(g[:, g_off + c]) in place; a [n, cols] contiguous, g 2-D rows of the same precision."""
+    _dev(a, g)
+    n, cols = a.shape
+    if g.dim() != 2 or g.shape[0] != n or g.dtype != a.dtype or g_off < 0 or g_off + cols > g.shape[1] or not a.is_contiguous():
+        raise KernelError(f"sigmoid_gate: a gate {tuple(g.shape)} {g.dtype} at {g_off} does not fit rows {tuple(a.shape)} {a.dtype}")
+    _check(library().ia_sigmoid_gate(_p(a), _p(g), n, cols, g.stride(0), g_off, _dt(a), _stream()))
+    return a
+
+
+def clamped_gate_mul(gu: torch.Tensor, limit: float, slope: float) -> torch.Tensor:
+    """Rows of [gate | up] -> g' * sigmoid(slope g') * (u' + 1) with g' = min(gate, limit), u' = clamp(up, -limit, limit)."""
+    _dev(gu)
+    n, two = gu.shape
+    if two % 2 or not gu.is_contiguous():
+        raise KernelError(f"clamped_gate_mul: rows {tuple(gu.shape)} are no [gate | up]")
+    out = torch.empty((n, two // 2), dtype=gu.dtype, device=gu.device)
+    _check(library().ia_clamped_gate_mul(_p(out), _p(gu), n, two // 2, ctypes.c_float(limit), ctypes.c_float(slope), _dt(gu),
+                                         _stream()))
+    return out
+
+
+def scale_inplace(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """x *= factor (32-bit values)."""
+    _dev(x); _f32(x, "x")
+    _check(library().ia_scale(_p(x), ctypes.c_longlong(x.numel()), ctypes.c_float(factor), _stream()))
+    return x

@@ -10,7 +10,12 @@ output projection.  q head h reads kv head h // (n_heads / n_kv_heads)
 Options of the spec beyond the reference's layer: biases, a window, a sink in the softmax (`sink`: the denominator
 holds one more term, exp(0)), values that are the key projection's own rows, ahead of norm and rotation (`values_from_keys`: no
 value projection is loaded; the key projection's rows stand twice in the fused product, so the kernels that take
-[q | k | v] serve unchanged), and other names for the tensors in the file (`names`).
+[q | k | v] serve unchanged), and other names for the tensors in the file (`names`).  Further: values of a width of
+their own (`v_head_dim`: the cache's value array, the heads' outputs and the output projection's input are that wide), a
+sigmoid gate on the joined heads (`gate`: sigmoid(W_g h), one product with the projections), and a layer without keys and
+values of its own (`own_kv` False: its stop of the schedule reads another stop's cache, after that layer's norm and
+rotation, with its own queries, window and scale).  Such a layer's rows are [q | k | v | g], whatever of these it has, and
+go through the kernels that take rows of any layout.
 """
 from __future__ import annotations
 
@@ -37,6 +42,8 @@ class Attention(Mixer):
         t = cls._tensors(spec)
         if spec.values_from_keys:
             t = {k: v for k, v in t.items() if not k.startswith("v_proj.")}
+        if not spec.own_kv:
+            t = {k: v for k, v in t.items() if not k.startswith(("k_proj.", "v_proj.", "k_norm."))}
         return {named.get(k, k): v for k, v in t.items()}
 
     @classmethod
@@ -45,23 +52,28 @@ class Attention(Mixer):
         t = {
             "q_proj.weight": TensorSpec((q_out, spec.hidden)),
             "k_proj.weight": TensorSpec((kv_out, spec.hidden)),
-            "v_proj.weight": TensorSpec((kv_out, spec.hidden)),
-            "o_proj.weight": TensorSpec((spec.hidden, q_out)),
+            "v_proj.weight": TensorSpec((spec.n_kv_heads * spec.value_dim, spec.hidden)),
+            "o_proj.weight": TensorSpec((spec.hidden, spec.n_heads * spec.value_dim)),
         }
+        if spec.gate:
+            t["g_proj.weight"] = TensorSpec((spec.n_heads * spec.value_dim, spec.hidden))
         if spec.qk_norm is not None:
             t["q_norm.weight"] = TensorSpec((spec.head_dim,), "norm")
             t["k_norm.weight"] = TensorSpec((spec.head_dim,), "norm")
         if spec.qkv_bias:
             t["q_proj.bias"] = TensorSpec((q_out,))
             t["k_proj.bias"] = TensorSpec((kv_out,))
-            t["v_proj.bias"] = TensorSpec((kv_out,))
+            t["v_proj.bias"] = TensorSpec((spec.n_kv_heads * spec.value_dim,))
         if spec.o_bias:
             t["o_proj.bias"] = TensorSpec((spec.hidden,))
         return t
 
     @classmethod
     def cache_need(cls, spec: AttentionSpec):
-        return PagedKV(spec.n_kv_heads, spec.head_dim, spec.window)
+        if not spec.own_kv:
+            return None
+        return PagedKV(spec.n_kv_heads, spec.head_dim, spec.kept_window,
+                       v_head_dim=spec.value_dim if spec.value_dim != spec.head_dim else None)
 
     def __init__(self, spec: AttentionSpec, tensors: Dict[str, torch.Tensor], dtype, device):
         if spec.n_heads % spec.n_kv_heads:
@@ -77,9 +89,21 @@ class Attention(Mixer):
             raise SpecError(f"attention: window {spec.window} must be >= 1")
         if spec.qk_norm is not None and spec.qk_norm.size != spec.head_dim:
             raise SpecError("attention: qk_norm must span head_dim")
+        if not (1 <= spec.value_dim <= 512):
+            raise SpecError(f"attention: v_head_dim {spec.value_dim} is outside 1..512, the range of the attention kernels")
+        if spec.values_from_keys and (spec.value_dim != spec.head_dim or not spec.own_kv):
+            raise SpecError("attention: values that are the keys have the keys' width and a key projection to come from")
         self.spec = spec
         named = dict(spec.names or ())
         tensors = {k: tensors[named.get(k, k)] for k in self._tensors(spec) if named.get(k, k) in tensors}
+        # rows of the plain layout [q | k | v], heads of one width, go through the kernels made for it; everything else
+        # (a gate in the rows, values of another width, no keys at all) through those that take any layout
+        self.plain = spec.own_kv and not spec.gate and spec.value_dim == spec.head_dim
+        if not self.plain:
+            if spec.qkv_bias:
+                raise SpecError("attention: biases go with rows of the plain layout [q | k | v]")
+            self._init_general(spec, tensors, dtype, device)
+            return
         if spec.values_from_keys:
             tensors["v_proj.weight"] = tensors["k_proj.weight"]
             if spec.qkv_bias:
@@ -98,10 +122,77 @@ class Attention(Mixer):
         if getattr(self.position, "magnitude", 1.0) != 1.0:
             raise SpecError("attention: a rotation law that scales cos and sin is not taken by this mixer's kernels")
 
+    def _init_general(self, spec: AttentionSpec, tensors, dtype, device):
+        H, G, d, dv = spec.n_heads, spec.n_kv_heads, spec.head_dim, spec.value_dim
+        stacked, at = [tensors["q_proj.weight"]], H * d
+        self.q_off, self.k_off, self.v_off, self.g_off = 0, None, None, None
+        if spec.own_kv:
+            stacked += [tensors["k_proj.weight"], tensors["v_proj.weight"]]
+            self.k_off, self.v_off, at = at, at + G * d, at + G * d + G * dv
+        if spec.gate:
+            stacked.append(tensors["g_proj.weight"])
+            self.g_off, at = at, at + H * dv
+        self.qkv = Linear(stacked, dtype, device)
+        self.o = Linear([tensors["o_proj.weight"]], dtype, device, [tensors["o_proj.bias"]] if spec.o_bias else None)
+        self.q_norm_w = self.k_norm_w = None
+        self.norm_eps, self.norm_add_one = 0.0, False
+        if spec.qk_norm is not None:
+            self.q_norm_w = tensors["q_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
+            if spec.own_kv:
+                self.k_norm_w = tensors["k_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
+            self.norm_eps, self.norm_add_one = float(spec.qk_norm.eps), bool(spec.qk_norm.add_one)
+        self.position = part_class("position", spec.position)(spec.position, {}, dtype, device)
+        if getattr(self.position, "magnitude", 1.0) != 1.0:
+            raise SpecError("attention: a rotation law that scales cos and sin is not taken by this mixer's kernels")
+
+    def _forward_general(self, ctx, h, cache):
+        s = self.spec
+        H, G, d, dv = s.n_heads, s.n_kv_heads, s.head_dim, s.value_dim
+        group = ctx.groups[cache.group]
+        if hasattr(h, "materialize"):
+            h = h.materialize()
+        proj = self.qkv(h)                                       # [n, q | k | v | g]
+        table = ctx.position_table(self.position)
+        cos, sin = table if table is not None else (None, None)
+        writes = cache.writable and s.own_kv
+        q = ops.qk_rope_kv_strided(
+            proj, H, G, d, dv, q_off=self.q_off, k_off=self.k_off if writes else None, v_off=self.v_off,
+            q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w, eps=self.norm_eps, add_one=self.norm_add_one, cos=cos, sin=sin,
+            rot=self.position.rot_dim, interleaved=self.position.interleaved, k_cache=cache.k, v_cache=cache.v,
+            slots=group.slots if writes else None, page_size=group.page_size)
+        a = self._attend(ctx, q, cache, group)
+        joined = a.view(a.shape[0], H * dv)
+        if s.gate:
+            ops.sigmoid_gate(joined, proj, self.g_off)
+        return self._project(ctx, joined)
+
+    def _attend(self, ctx, q, cache, group):
+        """The paged attention of the step's queries: the matrix cores where they take the sizes, else the plain kernel."""
+        s = self.spec
+        if ops.attention_mfma_fits(q.dtype, s.head_dim, group.page_size, s.value_dim):
+            common = dict(window=s.window, scale=s.softmax_scale, sink=s.sink)
+            if 0 < ctx.n_single < ctx.n_seqs:
+                # single tokens (decode) and portions of prompts want different launches: the first
+                # split their long key ranges between waves, the second have columns enough
+                a = ops.attention_mfma(q, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table,
+                                       max_q_len=1, max_kv_len=ctx.max_kv_single, seqs=(0, ctx.n_single),
+                                       tokens=(0, ctx.n_single), **common)
+                ops.attention_mfma(q, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table,
+                                   max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_multi,
+                                   seqs=(ctx.n_single, ctx.n_seqs - ctx.n_single),
+                                   tokens=(ctx.n_single, ctx.n_tokens - ctx.n_single), out=a, **common)
+                return a
+            return ops.attention_mfma(q, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table,
+                                      max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len, **common)
+        return ops.attention_generic(q, cache.k, cache.v, ctx.positions, ctx.token_seq, group.block_table,
+                                     window=s.window, scale=s.softmax_scale, max_kv_len=ctx.max_kv_len, sink=s.sink)
+
     def load_notes(self, page_size: int):
         """What the log should say once when a model with this part is set up: a decode step that cannot take the
         fused kernel still runs, three kernels where one would do."""
         dtype = self.qkv.weight.dtype
+        if not self.plain:
+            return []
         has_rotation = self.position.rot_dim > 0
         if dtype != torch.bfloat16 or ops.attention_decode_fused_fits(dtype, self.spec.head_dim, page_size,
                                                                       self.position.rot_dim, self.position.interleaved,
@@ -127,6 +218,8 @@ class Attention(Mixer):
         return self.o(a)
 
     def forward(self, ctx, h, cache):
+        if not self.plain:
+            return self._forward_general(ctx, h, cache)
         s = self.spec
         group = ctx.groups[cache.group]
         qkv = self.qkv(h)

@@ -5,7 +5,12 @@ W_down (g * sigmoid(alpha g) * (u + 1)).  The router's logits are 32-bit.
 `forward` returns `RoutedRows`: one 32-bit output row a (token, chosen expert) and the weights; whoever adds the
 feed-forward's output to the stream adds them up, a token's rows in the order of its choice, so a token's sum does
 not depend on the other tokens of the step (`.materialize()` gives the plain sum for a block that knows nothing of
-this)."""
+this).
+
+Options of the spec: `identity` more outputs of the router behind the experts', each standing for an expert that hands
+its input on (no tensors: `RoutedRows.sel` and `.real_experts` tell whoever adds the rows up which pairs these are, and
+the stream's own row takes their place); `correction`, a vector added to the scores for the choice only; `shared`, a
+feed-forward of the experts' form that runs for every token (`ClampedMlp`; its output rides along as `RoutedRows.extra`)."""
 from __future__ import annotations
 
 from typing import Dict
@@ -13,20 +18,25 @@ from typing import Dict
 import torch
 
 from .. import ops
-from ..config.spec import RoutedExpertsSpec, SpecError
+from ..config.spec import ClampedMlpSpec, RoutedExpertsSpec, SpecError
 from ..weights.loader import TensorSpec
-from .base import FeedForward, register_ffn
-from .linear import to_compute
+from .base import FeedForward, part_class, register_ffn
+from .linear import Linear, to_compute
 
 
 class RoutedRows:
-    """rows [n, top, width] (32-bit) and weights [n, top] (32-bit): the output is sum_k weights[:, k] * rows[:, k]."""
-    __slots__ = ("rows", "weights")
+    """rows [n, top, width] (32-bit) and weights [n, top] (32-bit): the output is sum_k weights[:, k] * rows[:, k].
+    `sel` [n, top] with `real_experts`: a pair whose choice is `real_experts` or more has no row here; the
+    feed-forward's own input stands for it.  `extra` [n, width]: a dense output to be added beside the rows."""
+    __slots__ = ("rows", "weights", "sel", "real_experts", "extra")
 
-    def __init__(self, rows: torch.Tensor, weights: torch.Tensor):
-        self.rows, self.weights = rows, weights
+    def __init__(self, rows: torch.Tensor, weights: torch.Tensor, sel=None, real_experts: int = 0, extra=None):
+        self.rows, self.weights, self.sel, self.real_experts, self.extra = rows, weights, sel, real_experts, extra
 
     def materialize(self) -> torch.Tensor:
+        if self.sel is not None or self.extra is not None:
+            raise SpecError("routed_experts: experts that hand their input on, and a shared expert, need a block "
+                            "arrangement that adds the routed rows up itself")
         n, top, width = self.rows.shape
         streams = torch.zeros((n, 1, width), dtype=torch.float32, device=self.rows.device)
         one = torch.ones((1,), dtype=torch.float32, device=self.rows.device)
@@ -40,7 +50,12 @@ class RoutedExperts(FeedForward):
 
     @classmethod
     def tensors(cls, spec: RoutedExpertsSpec) -> Dict[str, TensorSpec]:
-        t = {"router": TensorSpec((spec.experts, spec.hidden))}
+        t = {"router": TensorSpec((spec.experts + spec.identity, spec.hidden))}
+        if spec.correction:
+            t["correction"] = TensorSpec((spec.experts + spec.identity,))
+        if spec.shared is not None:
+            for local, ts in part_class("ffn", spec.shared).tensors(spec.shared).items():
+                t["shared." + local] = ts
         for e in range(spec.experts):
             t[f"e{e}.gate"] = TensorSpec((spec.intermediate, spec.hidden))
             t[f"e{e}.up"] = TensorSpec((spec.intermediate, spec.hidden))
@@ -48,13 +63,22 @@ class RoutedExperts(FeedForward):
         return t
 
     def __init__(self, spec: RoutedExpertsSpec, tensors: Dict[str, torch.Tensor], dtype, device):
-        if not (1 <= spec.top <= spec.experts <= ops.mix.MAX_EXPERTS) or spec.top > ops.mix.MAX_TOP:
-            raise SpecError(f"routed_experts: top {spec.top} of {spec.experts} experts (up to {ops.mix.MAX_TOP} of {ops.mix.MAX_EXPERTS})")
+        outputs = spec.experts + spec.identity
+        if (not (1 <= spec.top <= outputs <= ops.mix.MAX_EXPERTS) or spec.top > ops.mix.MAX_TOP or spec.experts < 1
+                or spec.identity < 0):
+            raise SpecError(f"routed_experts: top {spec.top} of {spec.experts} experts and {spec.identity} that hand their "
+                            f"input on (up to {ops.mix.MAX_TOP} of {ops.mix.MAX_EXPERTS})")
         if spec.score not in ops.mix.SCORE_FUNCTIONS:
             raise SpecError(f"routed_experts: score {spec.score!r} has no kernel (known: {sorted(ops.mix.SCORE_FUNCTIONS)})")
         self.spec = spec
         # the router's logits are 32-bit sums whatever its matrix is stored in (`ops.route`)
         self.router = to_compute(tensors["router"], dtype, device)
+        self.correction = (tensors["correction"].to(device=device, dtype=torch.float32).contiguous()
+                           if spec.correction else None)
+        self.shared = None
+        if spec.shared is not None:
+            self.shared = part_class("ffn", spec.shared)(
+                spec.shared, {k[len("shared."):]: v for k, v in tensors.items() if k.startswith("shared.")}, dtype, device)
         E = spec.experts
         gate_up = torch.stack([torch.cat([to_compute(tensors[f"e{e}.gate"], dtype, device),
                                           to_compute(tensors[f"e{e}.up"], dtype, device)], dim=0) for e in range(E)])
@@ -68,6 +92,34 @@ class RoutedExperts(FeedForward):
 
     def forward(self, ctx, h):
         s = self.spec
-        sel, weights = ops.route(h, self.router, s.top, s.scale, s.score, s.renormalize)
-        return RoutedRows(ops.experts_forward(h, sel, self.gate_up, self.down, s.limit, s.alpha,
-                                              ff=s.intermediate if self.tiled else None), weights)
+        sel, weights = ops.route(h, self.router, s.top, s.scale, s.score, s.renormalize, self.correction)
+        rows = ops.experts_forward(h, sel, self.gate_up, self.down, s.limit, s.alpha,
+                                   ff=s.intermediate if self.tiled else None)
+        extra = self.shared.forward(ctx, h) if self.shared is not None else None
+        if s.identity == 0 and extra is None:
+            return RoutedRows(rows, weights)
+        return RoutedRows(rows, weights, sel if s.identity else None, s.experts, extra)
+
+
+@register_ffn("clamped_mlp")
+class ClampedMlp(FeedForward):
+    """A gated feed-forward in the form of a routed expert, for every token: W_down (g' * sigmoid(alpha g') * (u' + 1)),
+    g' = min(W_gate h, limit), u' = clamp(W_up h, -limit, limit).  Gate and up share one product."""
+    graph_safe = True
+
+    @classmethod
+    def tensors(cls, spec: ClampedMlpSpec) -> Dict[str, TensorSpec]:
+        return {"gate": TensorSpec((spec.intermediate, spec.hidden)), "up": TensorSpec((spec.intermediate, spec.hidden)),
+                "down": TensorSpec((spec.hidden, spec.intermediate))}
+
+    def __init__(self, spec: ClampedMlpSpec, tensors: Dict[str, torch.Tensor], dtype, device):
+        if not spec.limit > 0:
+            raise SpecError(f"clamped_mlp: limit {spec.limit} must be positive")
+        self.spec = spec
+        self.gate_up = Linear([tensors["gate"], tensors["up"]], dtype, device)
+        self.down = Linear([tensors["down"]], dtype, device)
+
+    def forward(self, ctx, h):
+        if hasattr(h, "materialize"):
+            h = h.materialize()
+        return self.down(ops.clamped_gate_mul(self.gate_up(h), self.spec.limit, self.spec.alpha))

@@ -27,7 +27,17 @@ class TableEmbedding(Embedding):
         self.table = to_compute(tensors[spec.name], dtype, device)
 
     def forward(self, ctx) -> torch.Tensor:
-        return ops.embed_gather(self.table, ctx.token_ids)
+        scale, wide = float(getattr(self.spec, "scale", 1.0)), bool(getattr(self.spec, "wide", False))
+        if wide:
+            # 32-bit rows for a stream that is kept so: the factor meets the table's values unrounded
+            if self.table.dtype == torch.float32:
+                return ops.embed_gather_scaled(self.table, ctx.token_ids, scale)
+            rows, ctx.post_rows = ops.embed_gather_scaled(self.table, ctx.token_ids, scale, rounded=True)
+            return rows
+        rows = ops.embed_gather(self.table, ctx.token_ids)
+        if scale != 1.0:
+            rows = ops.embed_gather_scaled(self.table, ctx.token_ids, scale).to(rows.dtype)
+        return rows
 
 
 @register_head("lm_head")
@@ -64,7 +74,9 @@ class LinearHead(Head):
             self.weight = table                      # logits share the embedding table
 
     def forward(self, rows: torch.Tensor) -> torch.Tensor:
-        return ops.linear(rows, self.weight, torch.float32)
+        logits = ops.linear(rows, self.weight, torch.float32)
+        scale = float(getattr(self.spec, "scale", 1.0))
+        return logits if scale == 1.0 else ops.scale_inplace(logits, scale)
 
 
 @register_head("capped_lm_head")

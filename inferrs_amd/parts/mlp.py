@@ -22,6 +22,11 @@ class GatedMlp(FeedForward):
 
     @classmethod
     def tensors(cls, spec: GatedMlpSpec) -> Dict[str, TensorSpec]:
+        named = dict(spec.names or ())
+        return {named.get(k, k): v for k, v in cls._tensors(spec).items()}
+
+    @classmethod
+    def _tensors(cls, spec: GatedMlpSpec) -> Dict[str, TensorSpec]:
         t = {
             "gate_proj.weight": TensorSpec((spec.intermediate, spec.hidden)),
             "up_proj.weight": TensorSpec((spec.intermediate, spec.hidden)),
@@ -37,6 +42,8 @@ class GatedMlp(FeedForward):
         if spec.activation not in ops.ACTIVATIONS:
             raise SpecError(f"gated_mlp: activation {spec.activation!r} has no kernel (known: {sorted(ops.ACTIVATIONS)})")
         self.spec = spec
+        named = dict(spec.names or ())
+        tensors = {k: tensors[named.get(k, k)] for k in self._tensors(spec) if named.get(k, k) in tensors}
         self.gate_up = Linear([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dtype, device,
                               [tensors["gate_proj.bias"], tensors["up_proj.bias"]] if spec.bias else None)
         self.down = Linear([tensors["down_proj.weight"]], dtype, device, [tensors["down_proj.bias"]] if spec.bias else None)
