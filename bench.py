@@ -18,10 +18,12 @@ choice): `mixed16` is 16 requests with prompts of 128 to 4,096 random tokens in 
 `--decode-tokens` tokens.  Its JSON line gives tokens a second over the whole run, the prompts' and the
 decoded tokens' rates apart, and the time to a request's first token.
 
-    python bench.py --design buketar|lofudra [--design-shapes 1k,2k,4k]
+    python bench.py --design buketar|lofudra|fisanex [--design-shapes 1k,2k,4k]
 
-measures the Buketar design (latent attention, gated recurrences, routed experts, residual streams) or the Lofudra
-design (windowed sink attention beside retention, matrix memory, state space, norms on both sides) at a few layer
+measures the Buketar design (latent attention, gated recurrences, routed experts, residual streams), the Lofudra
+design (windowed sink attention beside retention, matrix memory, state space, norms on both sides) or the Fisanex design
+(a stream normed after every sum, gated window attention with values narrower than keys over caches that layers share,
+routed experts with outputs that hand the input on and a shared expert) at a few layer
 sizes beside the dense decoder at equal width, layers and feed-forward products a token: prompts of `--prefill-tokens`
 tokens, decode steps at `--batch` and at batch 1 through the serving loop, and every kernel's time in one prompt and one
 decode step of both.  One JSON line; the default record above is not touched by it.
@@ -421,17 +423,59 @@ LOFUDRA_LIKE_KERNEL = {"sandwich_step": "add_rmsnorm", "activation": "gate_mul",
                        "linear_scan": "attention_mfma", "linear_scan_chunked": "attention_mfma"}
 
 
+# ---- the Fisanex design beside the dense decoder at equal size (`--design fisanex`) ---------------------------
+# Layer sizes in the range of real models of its kind: heads with keys of 128 and values of 64 over a window of 1,024, a
+# quarter as many key heads, half of a head turning; every other layer reads the keys and values of the layer before it
+# and has routed experts (32 and 4 outputs that hand the input on, 4 a token, a shared expert of twice their size)
+# where the layers with keys of their own have a gated feed-forward of 3 x width.  The dense twin has the same width and
+# number of layers, as many attention heads of size 128, and a gated feed-forward of 3 x width in every layer.
+def fisanex_shape(width: int, layers: int, vocab: int = 32768):
+    heads = width // 128
+    mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 64, "scale": 128 ** -0.5,
+             "mask": {"size": 1024}, "rot": {"base": 500000.0, "dims": 64}}
+    ff = 3 * width // 4 // 64 * 64
+    moe = {"kind": "moe", "router": {"experts": 32, "identity": 4, "top": 4}, "expert": {"ff": ff, "limit": 7.0},
+           "shared": {"ff": 2 * ff, "limit": 7.0}}
+    out = []
+    for i in range(layers):
+        if i % 2 == 0:
+            out.append({"type": "attention", "mixer": dict(mixer), "mlp": {"kind": "dense", "ff": 3 * width}})
+        else:
+            out.append({"type": "attention", "mixer": dict(mixer, kv_from=i - 1), "mlp": moe})
+    return {"architecture": "Fisanex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "postln_alpha": 2.0,
+            "embedding": {"scale": 8.0}, "logit_scale": 0.5, "layers": out}
+
+
+FISANEX_SHAPES = {"1k": dict(width=1024, layers=12), "2k": dict(width=2048, layers=12), "4k": dict(width=4096, layers=6)}
+
+
+def fisanex_twin(b: dict, vocab: int = 32768) -> dict:
+    return dict(QWEN3_8B, vocab_size=vocab, hidden_size=b["width"], intermediate_size=3 * b["width"],
+                num_hidden_layers=b["layers"], num_attention_heads=b["width"] // 128, num_key_value_heads=max(1, b["width"] // 512),
+                tie_word_embeddings=True)
+
+
+FISANEX_LIKE_KERNEL = {"postnorm_step": "add_rmsnorm", "qk_rope_kv_strided": "qk_rope_kv", "sigmoid_gate": "gate_mul",
+                       "clamped_gate_mul": "gate_mul", "embed_gather_scaled": "embed_gather", "scale": "rmsnorm",
+                       "experts_gate_up": "vendor_gemm", "experts_down": "vendor_gemm", "route": "rmsnorm",
+                       "route_plan": "rmsnorm", "attention_mfma": "attention_mfma"}
+
+
 def design_main(args) -> int:
     """Prefill and decode throughput of a design at a few layer sizes beside the dense decoder at equal
     size (random weights), and the time of every kernel of one prefill and one decode step of both."""
     import torch
     from inferrs_amd.config import Qwen3Config
     from inferrs_amd.config.buketar import BuketarConfig
+    from inferrs_amd.config.fisanex import FisanexConfig
     from inferrs_amd.config.lofudra import LofudraConfig
     from inferrs_amd.engine import Engine
     batch, context, prompt = args.batch, min(args.context, 2048), args.prefill_tokens
     records = {}
-    if args.design == "lofudra":
+    if args.design == "fisanex":
+        shapes, shape_of, twin_of, config_cls, like = FISANEX_SHAPES, fisanex_shape, fisanex_twin, FisanexConfig, FISANEX_LIKE_KERNEL
+        title, beside = "Fisanex", "Qwen3 dense at equal width and layers, heads of 128 and a feed-forward of 3 x width"
+    elif args.design == "lofudra":
         shapes, shape_of, twin_of, config_cls, like = LOFUDRA_SHAPES, lofudra_shape, lofudra_twin, LofudraConfig, LOFUDRA_LIKE_KERNEL
         title, beside = "Lofudra", "Qwen3 dense at equal width, layers and feed-forward products a token"
     else:
@@ -498,7 +542,7 @@ def main() -> int:
                     help="workloads: cut prompt portions so that a step's tokens are a multiple of this (0: off)")
     ap.add_argument("--decode-run", type=int, default=8,
                     help="decode steps that the serving loop queues on the GPU at once (1: one at a time)")
-    ap.add_argument("--design", default=None, choices=["buketar", "lofudra"],
+    ap.add_argument("--design", default=None, choices=["buketar", "lofudra", "fisanex"],
                     help="instead of the headline: prefill and decode throughput of this design at a few layer sizes "
                          "beside the dense decoder at equal size, with every kernel's time")
     ap.add_argument("--design-shapes", default=None, help="with --design: the sizes to run, with commas (default: all)")

@@ -260,6 +260,7 @@ int ia_group_norm_gate(void* out, const float* o, const float* den, const float*
 
 // Built per head size (-DIA_HEAD_DIM) into a library of its own.
 int ia_attention_mfma_head_dim(void);
+int ia_attention_mfma_value_dim(void);     // the values' width this library was built for (IA_VALUE_DIM; the keys' unless given)
 long long ia_attention_mfma_workspace(int n, int nq, int splits);
 int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_cache,
                       const void* v_cache, const int* block_table, const int* cu_tokens,

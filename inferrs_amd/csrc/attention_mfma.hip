@@ -41,16 +41,25 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define HD IA_HEAD_DIM
-#define DB (HD / 16)            // 16-dim blocks of the output
+// The values' width where it is not the keys' (IA_VALUE_DIM, a multiple of 16 up to 256): the kernel of single waves
+// and the merges of split keys take it; the decode kernel and the tile kernel are for values as wide as keys.
+#ifndef IA_VALUE_DIM
+#define IA_VALUE_DIM IA_HEAD_DIM
+#endif
+static_assert(IA_VALUE_DIM % 16 == 0 && IA_VALUE_DIM >= 16 && IA_VALUE_DIM <= 256, "value size");
+#define HDV IA_VALUE_DIM
+#define HDMAX (HD > HDV ? HD : HDV)
+#define DBV (HDV / 16)          // 16-dim blocks of the output
+#define DB (HD / 16)            // the same in the kernels for values as wide as keys
 #define KS ((HD + 31) / 32)     // 32-dim steps of the first product
 
 struct AttnParams {
-    bf16_t* out;                // [n, nq, d]
-    float* part_o;              // [n, nq, splits, d]   when splits > 1
+    bf16_t* out;                // [n, nq, dv]
+    float* part_o;              // [n, nq, splits, dv]  when splits > 1
     float* part_ml;             // [n, nq, splits, 2]   running maximum (log2 domain) and sum
     const bf16_t* q;            // [n, nq, d]
     const bf16_t* k_cache;      // [pages, nkv, page, d]
-    const bf16_t* v_cache;      // [pages, nkv, d, page]
+    const bf16_t* v_cache;      // [pages, nkv, dv, page]
     bf16_t* k_cache_w;          // the same arrays for the fused form's writes
     bf16_t* v_cache_w;
     const int* block_table;     // [seqs, max_pages]
@@ -116,14 +125,14 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         }
     }
 
-    f32x4 acc[NB][DB];
+    f32x4 acc[NB][DBV];
     float m[NB], l[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         m[nb] = -INFINITY;
         l[nb] = 0.f;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) acc[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int db = 0; db < DBV; ++db) acc[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
 
     const int window_floor = p.window > 0 ? (pmin - p.window + 1 > 0 ? pmin - p.window + 1 : 0) : 0;   // first key any column sees
@@ -139,7 +148,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
     // ---- operands of a step: 32 keys = two 16-slot halves, each inside one page --------------
     struct Operands {
         uint4 k[2][KS];         // tile t, dim step ks: row r <-> key k0 + 8*(r/4) + 4t + r%4
-        uint4 v[DB];            // dim block db: row r <-> dim 16 db + r, keys k0 + 8G .. +7
+        uint4 v[DBV];            // dim block db: row r <-> dim 16 db + r, keys k0 + 8G .. +7
     };
     // A step's 32 keys are two groups of 16 slots, each inside one page (page sizes are multiples of
     // 16): a Place says where a group lies, and moves on without a division.
@@ -164,8 +173,8 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
             const int page_a = bt[at.idx], page_b = bt[next.idx];
             const char* ka = (const char*)(p.k_cache + (((size_t)page_a * p.nkv + kvh) * p.page + at.off) * HD);
             const char* kb = (const char*)(p.k_cache + (((size_t)page_b * p.nkv + kvh) * p.page + next.off) * HD);
-            const char* va = (const char*)(p.v_cache + ((size_t)page_a * p.nkv + kvh) * HD * p.page + at.off);
-            const char* vb = (const char*)(p.v_cache + ((size_t)page_b * p.nkv + kvh) * HD * p.page + next.off);
+            const char* va = (const char*)(p.v_cache + ((size_t)page_a * p.nkv + kvh) * HDV * p.page + at.off);
+            const char* vb = (const char*)(p.v_cache + ((size_t)page_b * p.nkv + kvh) * HDV * p.page + next.off);
             const char* kbase = k_second ? kb : ka;
             const char* vbase = (v_second ? vb : va) + v_lane;
 #pragma unroll
@@ -174,7 +183,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
                 for (int ks = 0; ks < KS; ++ks)
                     op.k[t][ks] = (ks * 32 + G * 8 < HD) ? *(const uint4*)(kbase + k_lane[t] + ks * 64) : zero4();
 #pragma unroll
-            for (int db = 0; db < DB; ++db) op.v[db] = *(const uint4*)(vbase + db * v_stride);
+            for (int db = 0; db < DBV; ++db) op.v[db] = *(const uint4*)(vbase + db * v_stride);
             return;
         }
         // The request's last step.  Rows past its length are read from its last written slot instead
@@ -196,9 +205,9 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         int vkey = k0 + 8 * G;
         vkey = vkey < kv_total ? vkey : (kv_total - 1) & ~7;
         const int vpage = vkey / p.page == idx_a ? page_a : page_b;
-        const bf16_t* vbase = p.v_cache + (((size_t)vpage * p.nkv + kvh) * HD + r) * p.page + vkey % p.page;
+        const bf16_t* vbase = p.v_cache + (((size_t)vpage * p.nkv + kvh) * HDV + r) * p.page + vkey % p.page;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) op.v[db] = *(const uint4*)(vbase + (size_t)db * 16 * p.page);
+        for (int db = 0; db < DBV; ++db) op.v[db] = *(const uint4*)(vbase + (size_t)db * 16 * p.page);
     };
     auto compute_step = [&](Operands& op, int k0) {
         const bool edge = k0 + 31 > pmin || (p.window > 0 && k0 < pmax - p.window + 1);
@@ -208,7 +217,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
             const int first_bad = kv_total - (k0 + 8 * G);          // keys >= this index are unwritten
             if (first_bad < 8) {
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
+                for (int db = 0; db < DBV; ++db) {
                     uint32_t w[4] = {op.v[db].x, op.v[db].y, op.v[db].z, op.v[db].w};
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
@@ -225,7 +234,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
             const int first_good = window_floor - (k0 + 8 * G);     // keys below this index are outside every window
             if (first_good > 0) {
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
+                for (int db = 0; db < DBV; ++db) {
                     uint32_t w[4] = {op.v[db].x, op.v[db].y, op.v[db].z, op.v[db].w};
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
@@ -283,13 +292,13 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
             // ---- O^T += V^T . P^T ----------------------------------------------------------
             if (__any(alpha != 1.0f)) {
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
+                for (int db = 0; db < DBV; ++db) {
                     acc[nb][db][0] *= alpha; acc[nb][db][1] *= alpha;
                     acc[nb][db][2] *= alpha; acc[nb][db][3] *= alpha;
                 }
             }
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
+            for (int db = 0; db < DBV; ++db)
                 acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                     __builtin_bit_cast(bf16x8, op.v[db]), __builtin_bit_cast(bf16x8, pb), acc[nb][db], 0, 0, 0);
         }
@@ -333,18 +342,18 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         const size_t row = (size_t)(t0 + tq[nb]) * p.nq + head[nb];
         if (p.splits == 1) {
             const float inv = 1.0f / (p.sink ? lt + exp2f(-m[nb]) : lt);
-            bf16_t* o = p.out + row * HD + 4 * G;
+            bf16_t* o = p.out + row * HDV + 4 * G;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
+            for (int db = 0; db < DBV; ++db) {
                 uint2 w;
                 w.x = pack_bf16x2(acc[nb][db][0] * inv, acc[nb][db][1] * inv);
                 w.y = pack_bf16x2(acc[nb][db][2] * inv, acc[nb][db][3] * inv);
                 *(uint2*)(o + 16 * db) = w;
             }
         } else {
-            float* o = p.part_o + (row * p.splits + split) * HD + 4 * G;
+            float* o = p.part_o + (row * p.splits + split) * HDV + 4 * G;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) *(f32x4*)(o + 16 * db) = acc[nb][db];
+            for (int db = 0; db < DBV; ++db) *(f32x4*)(o + 16 * db) = acc[nb][db];
             if (G == 0) {
                 float* ml = p.part_ml + (row * p.splits + split) * 2;
                 ml[0] = m[nb];
@@ -359,7 +368,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
 // pair walks about the same number, so all waves end together.  It pays when the step's queries
 // span most of the context; a short portion late in a long context has equal blocks already.
 template <int NB>
-__global__ __launch_bounds__(IA_WAVE) __attribute__((amdgpu_waves_per_eu(HD <= 128 ? 2 : 1, HD > 64 ? 2 : 8)))
+__global__ __launch_bounds__(IA_WAVE) __attribute__((amdgpu_waves_per_eu(HDMAX <= 128 ? 2 : 1, HDMAX > 64 ? 2 : 8)))
 void attn_mfma_kernel(const AttnParams p) {
     const int kvh = blockIdx.y / p.splits, split = blockIdx.y - kvh * p.splits;
     const int seq = p.seq_begin + blockIdx.z;
@@ -437,7 +446,7 @@ struct DecodeOperands {
     uint4 v[DB];
 };
 
-template <bool ENABLED = (HD % 64 == 0)>
+template <bool ENABLED = (HD % 64 == 0 && HDV == HD)>
 __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnParams p, int* counters, int team) {
     if constexpr (ENABLED) {
         extern __shared__ __align__(16) float team_mem[];       // [team][columns][HD] partial outputs, then [team][columns][2]
@@ -966,7 +975,7 @@ __device__ __forceinline__ void lds_load16(const char* from, uint32_t lds_at) {
 #define TILE_NBW 2
 // NBW_: column tiles of 16 a wave.  One instead of two halves a block's columns (64) and doubles the blocks: for steps
 // whose blocks of 128 columns would leave compute units without one (short prompts, few heads).
-template <bool ENABLED = (HD == 128), int NBW_ = TILE_NBW>
+template <bool ENABLED = (HD == 128 && HDV == HD), int NBW_ = TILE_NBW>
 __global__ __launch_bounds__(TILE_GROUPS * TILE_WAVES * IA_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attn_tile_kernel(const AttnParams p) {
     if constexpr (ENABLED) {
@@ -1408,14 +1417,14 @@ static int attn_cus() {
 __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
     bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
     size_t first_row, int sink) {
-    constexpr int PER = (HD + IA_WAVE - 1) / IA_WAVE;
+    constexpr int PER = (HDV + IA_WAVE - 1) / IA_WAVE;
     __shared__ float weight[256];
     __shared__ float red[MERGE_WAVES][PER * IA_WAVE];
     __shared__ float s_total;
     const size_t row = first_row + blockIdx.x;
     const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
     const float* ml = part_ml + row * splits * 2;
-    const float* po = part_o + row * splits * HD;
+    const float* po = part_o + row * splits * HDV;
     // this wave's partial outputs, asked for before anything is waited for
     float v[256 / MERGE_WAVES][PER];
 #pragma unroll
@@ -1424,7 +1433,7 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
 #pragma unroll
         for (int t = 0; t < PER; ++t) {
             const int e = lane + t * IA_WAVE;
-            v[i][t] = (s < splits && e < HD) ? po[(size_t)s * HD + e] : 0.f;
+            v[i][t] = (s < splits && e < HDV) ? po[(size_t)s * HDV + e] : 0.f;
         }
     }
     if (wave == 0) {
@@ -1464,12 +1473,12 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
         const int e = lane + t * IA_WAVE;
         float sum = red[0][e];
         for (int w = 1; w < MERGE_WAVES; ++w) sum += red[w][e];
-        if (e < HD) out[row * HD + e].bits = f32_to_bf16_bits(sum * inv);
+        if (e < HDV) out[row * HDV + e].bits = f32_to_bf16_bits(sum * inv);
     }
 }
 
 // The same merge for steps with many rows and few splits (portions of prompts, decode steps of many
-// requests): a wave a row, every lane with the splits' maxima and sums of its row and HD / 64 features.
+// requests): a wave a row, every lane with the splits' maxima and sums of its row and HDV / 64 features.
 // Kernel times at head size 128, context 8,192, 32 heads (the block-a-row kernel against this one):
 // 512 rows of 8 splits 4.9 against 7.6 us, 1,024 rows of 4 splits 7.0 against 5.1, 2,048 rows of 4 splits
 // 12.2 against 5.0.
@@ -1478,13 +1487,13 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
 __global__ __launch_bounds__(MERGE_ROWS_WAVES * IA_WAVE) void attn_merge_rows_kernel(
     bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
     size_t first_row, size_t n_rows, int sink) {
-    constexpr int PER = (HD + IA_WAVE - 1) / IA_WAVE;
+    constexpr int PER = (HDV + IA_WAVE - 1) / IA_WAVE;
     const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
     const size_t local = (size_t)blockIdx.x * MERGE_ROWS_WAVES + wave;
     if (local >= n_rows) return;
     const size_t row = first_row + local;
     const float* ml = part_ml + row * splits * 2;
-    const float* po = part_o + row * splits * HD;
+    const float* po = part_o + row * splits * HDV;
     float mx = -INFINITY;
     for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ml[2 * s]);
     float total = 0.f, o[PER];
@@ -1497,22 +1506,23 @@ __global__ __launch_bounds__(MERGE_ROWS_WAVES * IA_WAVE) void attn_merge_rows_ke
 #pragma unroll
         for (int t = 0; t < PER; ++t) {
             const int e = lane + t * IA_WAVE;
-            if (e < HD) o[t] = fmaf(po[(size_t)s * HD + e], w, o[t]);
+            if (e < HDV) o[t] = fmaf(po[(size_t)s * HDV + e], w, o[t]);
         }
     }
     const float inv = 1.0f / (sink ? total + exp2f(-mx) : total);
 #pragma unroll
     for (int t = 0; t < PER; ++t) {
         const int e = lane + t * IA_WAVE;
-        if (e < HD) out[row * HD + e].bits = f32_to_bf16_bits(o[t] * inv);
+        if (e < HDV) out[row * HDV + e].bits = f32_to_bf16_bits(o[t] * inv);
     }
 }
 
 extern "C" int ia_attention_mfma_head_dim(void) { return HD; }
+extern "C" int ia_attention_mfma_value_dim(void) { return HDV; }
 
 // Floats of workspace that `splits` > 1 needs: partial outputs, then maxima and sums.
 extern "C" long long ia_attention_mfma_workspace(int n, int nq, int splits) {
-    return splits > 1 ? (long long)n * nq * splits * (HD + 2) : 0;
+    return splits > 1 ? (long long)n * nq * splits * (HDV + 2) : 0;
 }
 
 // The requests seq_begin .. seq_begin + n_seqs of the step, whose tokens are token_begin ..
@@ -1573,7 +1583,7 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
     AttnParams p;
     p.out = (bf16_t*)out;
     p.part_o = workspace;
-    p.part_ml = workspace ? workspace + (size_t)n * nq * splits * HD : nullptr;
+    p.part_ml = workspace ? workspace + (size_t)n * nq * splits * HDV : nullptr;
     p.q = (const bf16_t*)q;
     p.k_cache = (const bf16_t*)k_cache;
     p.v_cache = (const bf16_t*)v_cache;
@@ -1597,8 +1607,8 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
     const long long col_blocks = (cols + 16 * nb - 1) / (16 * nb);
     const dim3 grid((unsigned)(p.pair ? (col_blocks + 1) / 2 : col_blocks), nkv * splits, n_seqs);
     if (fused != nullptr) {
-        IA_CHECK(HD % 64 == 0 && max_q_len == 1, "attention_mfma: the fused form takes single tokens and head sizes in "
-                 "steps of 64 (head size %d, %d tokens a request)", HD, max_q_len);
+        IA_CHECK(HD % 64 == 0 && HDV == HD && max_q_len == 1, "attention_mfma: the fused form takes single tokens, head sizes in "
+                 "steps of 64 and values as wide as keys (head size %d, %d tokens a request)", HD, max_q_len);
         p.qkv = (const bf16_t*)fused->qkv;
         p.q_norm_w = fused->q_norm_w; p.k_norm_w = fused->k_norm_w;
         p.cos_t = fused->cos_t; p.sin_t = fused->sin_t; p.slots = fused->slots;
@@ -1619,7 +1629,7 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         attn_decode_kernel<><<<fgrid, team * IA_WAVE, shared, stream>>>(p, fused->counters, team);
         IA_LAUNCH_CHECK("attention_decode");
         return 0;
-    } else if (HD == 128 && g_tiles && cols >= 16 * TILE_NBW * TILE_WAVES && (splits == 1 || chunk % TILE_STAGE == 0)) {
+    } else if (HD == 128 && HDV == HD && g_tiles && cols >= 16 * TILE_NBW * TILE_WAVES && (splits == 1 || chunk % TILE_STAGE == 0)) {
         // portions of prompts: blocks of four waves that share the keys through shared memory
         // Blocks of 128 columns; of 64 (twice as many, the same bits) where the keys are not split and the blocks of 128
         // would be half a compute unit's worth or less, or, under a causal mask over most of the context, where the
@@ -1637,7 +1647,7 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         IA_CHECK(tiles <= 65535, "attention_mfma: %lld tiles of columns in a request (at most 65535)", tiles);
         const dim3 tgrid((unsigned)(nkv * splits * n_seqs), (unsigned)tiles, 1);
         p.pair = 0;
-        if (narrow) attn_tile_kernel<(HD == 128), 1><<<tgrid, TILE_GROUPS * TILE_WAVES * IA_WAVE, 0, stream>>>(p);
+        if (narrow) attn_tile_kernel<(HD == 128 && HDV == HD), 1><<<tgrid, TILE_GROUPS * TILE_WAVES * IA_WAVE, 0, stream>>>(p);
         else attn_tile_kernel<><<<tgrid, TILE_GROUPS * TILE_WAVES * IA_WAVE, 0, stream>>>(p);
     } else if (nb == 1) {
         attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);
@@ -1671,7 +1681,7 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
 }
 
 // Whether this head size has the fused decode form.
-extern "C" int ia_attention_mfma_has_fused(void) { return HD % 64 == 0 ? 1 : 0; }
+extern "C" int ia_attention_mfma_has_fused(void) { return HD % 64 == 0 && HDV == HD ? 1 : 0; }
 
 // Decode steps, one token a request: the per-head norm of q and k (weights may be null: none), the rotation
 // by each token's angles (cos, sin [n, d / 2], whole heads, halves paired; may be null: none) and the write

@@ -437,7 +437,7 @@ ATTN_MIN_CHUNK = 64            # fewest keys a split is worth
 def attention_mfma_fits(dtype: torch.dtype, d: int, page_size: int, dv: Optional[int] = None) -> bool:
     """`dv`: the values' width where it is not the keys'."""
     return (dtype == torch.bfloat16 and d in _build.ATTN_HEAD_DIMS and page_size % 16 == 0
-            and (dv is None or dv == d))
+            and (dv is None or dv in _build.ATTN_HEAD_DIMS))
 
 
 ATTN_TILE_COLS = 128           # head size 128, prompt portions: columns a block of four waves
@@ -516,8 +516,9 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     _i32(positions, "positions"); _i32(cu_tokens, "cu_tokens"); _i32(block_table, "block_table")
     n, nq, d = q.shape
     nkv, page_size = k_cache.shape[1], k_cache.shape[2]
-    _check_cache(k_cache, v_cache, nkv, page_size, d, q.dtype, "attention")
-    if not attention_mfma_fits(q.dtype, d, page_size):
+    dv = v_cache.shape[2] if v_cache.dim() == 4 else d
+    _check_cache(k_cache, v_cache, nkv, page_size, d, q.dtype, "attention", dv)
+    if not attention_mfma_fits(q.dtype, d, page_size, dv):
         raise KernelError(f"attention_mfma: takes bfloat16, head sizes {_build.ATTN_HEAD_DIMS[0]}.."
                           f"{_build.ATTN_HEAD_DIMS[-1]} in steps of 16 and page sizes in steps of 16; got "
                           f"{q.dtype}, head size {d}, page size {page_size}")
@@ -531,14 +532,15 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         raise KernelError(f"attention_mfma: max_kv_len {max_kv_len} / max_q_len {max_q_len} do not fit "
                           f"{block_table.shape[1]} pages of {page_size} and {n_tokens} tokens")
     if out is None:
-        out = torch.empty_like(q)
-    elif out.shape != q.shape or out.dtype != q.dtype:
-        raise KernelError("attention_mfma: `out` must have the shape and dtype of q")
+        out = torch.empty((n, nq, dv), dtype=q.dtype, device=q.device)
+    elif tuple(out.shape) != (n, nq, dv) or out.dtype != q.dtype:
+        raise KernelError("attention_mfma: `out` must be [n, nq, the values' width] in the dtype of q")
     if splits is None:
-        splits, chunk = attention_split(n_seqs, nkv, nq // nkv, max_q_len, max_kv_len, d)
+        # (values of a width of their own stay on the kernel of single waves: its rule for splitting the keys)
+        splits, chunk = attention_split(n_seqs, nkv, nq // nkv, max_q_len, max_kv_len, d if dv == d else 0)
     else:
         chunk = -(-(-(-max_kv_len // splits)) // 64) * 64
-    target = _build.attn_target(d)
+    target = _build.attn_target(d, dv)
     lib = library(target)
     ws_floats = lib.ia_attention_mfma_workspace(n, nq, splits)
     ws = torch.empty((ws_floats,), dtype=torch.float32, device=q.device) if ws_floats else None

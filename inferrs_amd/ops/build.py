@@ -3,7 +3,8 @@
 Three kinds of library:
   * "core": every HIP kernel (gfx950) whose code does not depend on a model size;
   * "attn_d<N>": the matrix-core attention kernel built for head size N (`-DIA_HEAD_DIM=N`),
-    so that a model compiles only the head size it has;
+    so that a model compiles only the head size it has; "attn_d<N>_v<M>" the same for values of
+    width M beside keys of width N (`-DIA_VALUE_DIM=M`), compiled when a model with such heads asks;
   * "runtime": the host runtime (cache manager, step assembly, scheduler), plain C++ that
     touches no GPU and is compiled with the host compiler.
 
@@ -46,14 +47,20 @@ SHARED = ("error.hip",)
 RUNTIME_SOURCES = ("runtime.cpp",)
 RUNTIME_HEADERS = ("runtime.h",)
 ATTN_HEAD_DIMS = tuple(range(16, 257, 16))
+# (keys' width, values' width) pairs that `build_all` compiles beside the head sizes (any other pair of ATTN_HEAD_DIMS is
+# compiled when it is first asked for)
+ATTN_VALUE_PAIRS = ((32, 48), (64, 16), (64, 256), (128, 64))
 
 
-def attn_target(head_dim: int) -> str:
-    return f"attn_d{head_dim}"
+def attn_target(head_dim: int, value_dim: Optional[int] = None) -> str:
+    if value_dim is None or value_dim == head_dim:
+        return f"attn_d{head_dim}"
+    return f"attn_d{head_dim}_v{value_dim}"
 
 
 def all_targets() -> List[str]:
-    return ["runtime", "core"] + [attn_target(d) for d in ATTN_HEAD_DIMS]
+    return (["runtime", "core"] + [attn_target(d) for d in ATTN_HEAD_DIMS]
+            + [attn_target(d, dv) for d, dv in ATTN_VALUE_PAIRS])
 
 
 def _is_host(target: str) -> bool:
@@ -68,10 +75,12 @@ def _plan(target: str) -> Tuple[List[str], List[str]]:
     if target == "core":
         return [os.path.join(CSRC, n) for n in names if n not in PER_HEAD_DIM], []
     if target.startswith("attn_d"):
-        d = int(target[len("attn_d"):])
-        if d not in ATTN_HEAD_DIMS:
-            raise ValueError(f"no matrix-core attention kernel for head size {d}")
-        return [os.path.join(CSRC, n) for n in PER_HEAD_DIM + SHARED], [f"-DIA_HEAD_DIM={d}"]
+        sizes = target[len("attn_d"):].split("_v")
+        d, dv = int(sizes[0]), int(sizes[-1])
+        if d not in ATTN_HEAD_DIMS or dv not in ATTN_HEAD_DIMS:
+            raise ValueError(f"no matrix-core attention kernel for head size {d} with values of {dv}")
+        defines = [f"-DIA_HEAD_DIM={d}"] + ([f"-DIA_VALUE_DIM={dv}"] if dv != d else [])
+        return [os.path.join(CSRC, n) for n in PER_HEAD_DIM + SHARED], defines
     raise ValueError(f"unknown kernel library {target!r}")
 
 

@@ -428,18 +428,32 @@ def test_greedy_generation_through_the_scheduler(models, name):
 
 
 def test_decode_steps_replayed_from_graphs(models):
-    """Generation in bfloat16 with the serving loop's graphs against the same engine without them: the same tokens."""
+    """Generation with the serving loop's graphs against the same engine without them.  32-bit: the same sums in the
+    same order, so the same tokens.  bfloat16: a graph's step sees its context bucket's width and an eager step the
+    longest request, so keys may be split between waves in another way; given tokens are fed and the logits compared."""
     from inferrs_amd.engine import Engine
+    from inferrs_amd.engine.engine import Entry
     from inferrs_amd.sampling import SamplingParams
     folder, cfg, tensors, reqs, ref = models[("D", 1.0)]
     prompts = [random_tokens(n, cfg["vocab"], 700 + n) for n in (33, 5, 120)]
     outs = []
     for graphs in (False, True):
-        eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=64, max_seqs=4, use_graphs=graphs)
+        eng = Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=64, max_seqs=4, use_graphs=graphs)
+        assert eng.use_graphs == graphs
         res = eng.generate(prompts, [SamplingParams.greedy(max_tokens=40, bypass_stop_tokens=True)] * 3, max_batch_size=3)
-        assert all(o.error is None for o in res)
+        assert all(o.error is None for o in res) and (eng.graph_replays > 20) == graphs
         outs.append([o.tokens for o in res])
     assert outs[0] == outs[1]
+    toks = reqs["r6"]                                    # 130 tokens: 90 as a prompt, 40 fed one by one
+    want = ref["r6"][89:]
+    scale = float(np.abs(ref["r6"]).max())
+    for graphs in (False, True):
+        eng = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=64, max_seqs=4, use_graphs=graphs)
+        rows = [eng.step([Entry("a", toks[:90], [89])])[0].clone()]
+        rows += [eng.step([Entry("a", [t], [0])])[0].clone() for t in toks[90:]]
+        assert (eng.graph_replays > 20) == graphs
+        err = float(np.abs(torch.stack(rows).cpu().numpy() - want).max()) / scale
+        assert err <= 3e-2, (graphs, err)
 
 
 def test_random_weights_engine_steps():
