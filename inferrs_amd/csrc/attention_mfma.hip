@@ -51,6 +51,9 @@ static_assert(IA_VALUE_DIM % 16 == 0 && IA_VALUE_DIM >= 16 && IA_VALUE_DIM <= 25
 #define HDMAX (HD > HDV ? HD : HDV)
 #define DBV (HDV / 16)          // 16-dim blocks of the output
 #define DB (HD / 16)            // the same in the kernels for values as wide as keys
+// The tile kernel (prompt portions, keys of 128) takes values of 32 to 128 in steps of 32: a load of 1 KiB brings 32 features
+// of 16 keys, and the groups' exchange at its end fits the stages up to the keys' own width.
+#define TILE_FITS (HD == 128 && HDV % 32 == 0 && HDV <= 128)
 #define KS ((HD + 31) / 32)     // 32-dim steps of the first product
 
 struct AttnParams {
@@ -965,7 +968,8 @@ __device__ __forceinline__ void lds_load16(const char* from, uint32_t lds_at) {
 #define TILE_GROUPS 2             // groups of such waves in a block: each with its own stages (see the kernel)
 #define TILE_STAGE 64
 #define TILE_K_BYTES (TILE_STAGE * HD * 2)
-#define TILE_BUF_BYTES (2 * TILE_K_BYTES)
+#define TILE_V_CHUNKS (HDV / 32)  // loads of 1 KiB that bring a group of 16 keys' values: 32 features each
+#define TILE_BUF_BYTES (TILE_K_BYTES + TILE_STAGE * HDV * 2)
 
 // Two column tiles of 16 a wave, two blocks a compute unit, two waves a SIMD.  (Four tiles a wave, so that every key and
 // value read out of shared memory serves twice as many products, take the registers of a whole SIMD; with the softmax of
@@ -975,7 +979,7 @@ __device__ __forceinline__ void lds_load16(const char* from, uint32_t lds_at) {
 #define TILE_NBW 2
 // NBW_: column tiles of 16 a wave.  One instead of two halves a block's columns (64) and doubles the blocks: for steps
 // whose blocks of 128 columns would leave compute units without one (short prompts, few heads).
-template <bool ENABLED = (HD == 128 && HDV == HD), int NBW_ = TILE_NBW>
+template <bool ENABLED = TILE_FITS, int NBW_ = TILE_NBW>
 __global__ __launch_bounds__(TILE_GROUPS * TILE_WAVES * IA_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attn_tile_kernel(const AttnParams p) {
     if constexpr (ENABLED) {
@@ -1051,14 +1055,14 @@ void attn_tile_kernel(const AttnParams p) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) qreg[nb][ks] = cvalid[nb] ? *(const uint4*)(qrow + ks * 32 + G * 8) : zero4();
         }
-        f32x4 acc[NBW][DB];
+        f32x4 acc[NBW][DBV];
         float m[NBW], l[NBW];
 #pragma unroll
         for (int nb = 0; nb < NBW; ++nb) {
             m[nb] = -INFINITY;
             l[nb] = 0.f;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) acc[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int db = 0; db < DBV; ++db) acc[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
 
         // ---- a stage on its way: wave w brings keys 16 w .. + 16 and features 32 w .. + 32 ----------
@@ -1098,13 +1102,13 @@ void attn_tile_kernel(const AttnParams p) {
         const uint32_t v_from = (uint32_t)(((lane >> 1) * p.page + v_half * 8) * 2);
         auto issue = [&](char* buf, int page, int off) {
             const char* krows = (const char*)(p.k_cache + (((size_t)page * p.nkv + kvh) * p.page + off) * HD);
-            const char* vrows = (const char*)(p.v_cache + ((size_t)page * p.nkv + kvh) * HD * p.page + off);
+            const char* vrows = (const char*)(p.v_cache + ((size_t)page * p.nkv + kvh) * HDV * p.page + off);
             const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)buf;
 #pragma unroll
             for (int c = 0; c < 4; ++c) lds_load16(krows + k_from[c], at + (16 * wave_s + 4 * c) * (HD * 2));
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
-                lds_load16(vrows + (size_t)c * 32 * p.page * 2 + v_from, at + TILE_K_BYTES + wave_s * (16 * HD * 2) + c * 1024);
+            for (int c = 0; c < TILE_V_CHUNKS; ++c)
+                lds_load16(vrows + (size_t)c * 32 * p.page * 2 + v_from, at + TILE_K_BYTES + wave_s * (16 * HDV * 2) + c * 1024);
         };
         // values of keys past the request's length may hold anything at all: a lane zeroes them in the
         // pieces that it brought itself, once they have arrived
@@ -1117,8 +1121,8 @@ void attn_tile_kernel(const AttnParams p) {
             const int first_good = kb < bfloor ? bfloor - mine : 0;
             if (first_bad >= 8 && first_good <= 0) return;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                uint4* at = (uint4*)(buf + TILE_K_BYTES + wave_s * (16 * HD * 2) + c * 1024 + lane * 16);
+            for (int c = 0; c < TILE_V_CHUNKS; ++c) {
+                uint4* at = (uint4*)(buf + TILE_K_BYTES + wave_s * (16 * HDV * 2) + c * 1024 + lane * 16);
                 const uint4 v = *at;
                 uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -1137,7 +1141,7 @@ void attn_tile_kernel(const AttnParams p) {
             for (int ks = 0; ks < KS; ++ks) k_at[ks] = (uint32_t)(kl * (HD * 2)) + (((uint32_t)(ks * 4 + G) ^ k_xor) * 16);
         }
         // values: group of 16 keys (G >> 1 of the step's two), feature row of 32 bytes, half G & 1
-        const uint32_t v_at = (uint32_t)((G >> 1) * (16 * HD * 2) + r * 32 + (G & 1) * 16);
+        const uint32_t v_at = (uint32_t)((G >> 1) * (16 * HDV * 2) + r * 32 + (G & 1) * 16);
         int page_l, off_l;
         auto stage = [&](int s, char* buf, char* other) __attribute__((always_inline)) {
             if (s >= stages) {                             // the other group has a stage more: its barrier is kept
@@ -1231,15 +1235,15 @@ void attn_tile_kernel(const AttnParams p) {
             auto rescale = [&](int nb, float alpha) {
                 if (__any(alpha != 1.0f)) {
 #pragma unroll
-                    for (int db = 0; db < DB; ++db) {
+                    for (int db = 0; db < DBV; ++db) {
                         acc[nb][db][0] *= alpha; acc[nb][db][1] *= alpha;
                         acc[nb][db][2] *= alpha; acc[nb][db][3] *= alpha;
                     }
                 }
             };
-            auto weighted = [&](int nb, const uint4 (&vop)[DB], const uint4& pb) {
+            auto weighted = [&](int nb, const uint4 (&vop)[DBV], const uint4& pb) {
 #pragma unroll
-                for (int db = 0; db < DB; ++db)
+                for (int db = 0; db < DBV; ++db)
                     acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                         __builtin_bit_cast(bf16x8, vop[db]), __builtin_bit_cast(bf16x8, pb), acc[nb][db], 0, 0, 0);
             };
@@ -1258,7 +1262,7 @@ void attn_tile_kernel(const AttnParams p) {
             };
             auto step = [&](auto edge_c, int u) {
                 const int k0 = kb + 32 * u;
-                uint4 vop[DB];
+                uint4 vop[DBV];
                 if constexpr (NBW == 1) {
                     // one column tile: nothing of its own to lay beside the softmax (the SIMD's other wave is)
                     f32x4 s0[2];
@@ -1266,8 +1270,8 @@ void attn_tile_kernel(const AttnParams p) {
                     float alpha0;
                     scores(0, s0);
 #pragma unroll
-                    for (int db = 0; db < DB; ++db)
-                        vop[db] = *(const uint4*)(buf + TILE_K_BYTES + u * (32 * HD * 2) + db * 512 + v_at);
+                    for (int db = 0; db < DBV; ++db)
+                        vop[db] = *(const uint4*)(buf + TILE_K_BYTES + u * (32 * HDV * 2) + db * 512 + v_at);
                     softmax(edge_c, 0, k0, s0, pb0, alpha0);
                     if (u == 0) read_keys(1);
                     rescale(0, alpha0);
@@ -1278,8 +1282,8 @@ void attn_tile_kernel(const AttnParams p) {
                 float alpha0, alpha1;
                 scores(0, s0);
 #pragma unroll
-                for (int db = 0; db < DB; ++db)
-                    vop[db] = *(const uint4*)(buf + TILE_K_BYTES + u * (32 * HD * 2) + db * 512 + v_at);
+                for (int db = 0; db < DBV; ++db)
+                    vop[db] = *(const uint4*)(buf + TILE_K_BYTES + u * (32 * HDV * 2) + db * 512 + v_at);
                 __builtin_amdgcn_sched_barrier(0);
                 scores(1, s1);
                 softmax(edge_c, 0, k0, s0, pb0, alpha0);
@@ -1337,7 +1341,7 @@ void attn_tile_kernel(const AttnParams p) {
 #pragma unroll
                 for (int nb = 0; nb < NBW; ++nb) {
 #pragma unroll
-                    for (int db = 0; db < DB; ++db) xacc[(nb * DB + db) * IA_WAVE + lane] = acc[nb][db];
+                    for (int db = 0; db < DBV; ++db) xacc[(nb * DBV + db) * IA_WAVE + lane] = acc[nb][db];
                     xml[nb * IA_WAVE + lane] = make_float2(m[nb], l[nb]);
                 }
             }
@@ -1352,8 +1356,8 @@ void attn_tile_kernel(const AttnParams p) {
                 l[nb] = l[nb] * mine_w + other.y * other_w;
                 m[nb] = top;
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    const f32x4 o = xacc[(nb * DB + db) * IA_WAVE + lane];
+                for (int db = 0; db < DBV; ++db) {
+                    const f32x4 o = xacc[(nb * DBV + db) * IA_WAVE + lane];
                     acc[nb][db][0] = acc[nb][db][0] * mine_w + o[0] * other_w;
                     acc[nb][db][1] = acc[nb][db][1] * mine_w + o[1] * other_w;
                     acc[nb][db][2] = acc[nb][db][2] * mine_w + o[2] * other_w;
@@ -1368,9 +1372,9 @@ void attn_tile_kernel(const AttnParams p) {
             const size_t row = (size_t)(t0 + tq[nb]) * p.nq + head[nb];
             if (p.splits == 1) {
                 const float inv = 1.0f / (p.sink ? lt + exp2f(-m[nb]) : lt);
-                bf16_t* o = p.out + row * HD + 4 * G;
+                bf16_t* o = p.out + row * HDV + 4 * G;
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
+                for (int db = 0; db < DBV; ++db) {
                     uint2 w;
                     w.x = pack_bf16x2(acc[nb][db][0] * inv, acc[nb][db][1] * inv);
                     w.y = pack_bf16x2(acc[nb][db][2] * inv, acc[nb][db][3] * inv);
@@ -1378,9 +1382,9 @@ void attn_tile_kernel(const AttnParams p) {
                 }
             } else {
                 // for the merge: sums and accumulators relative to the exponents' reference point m
-                float* o = p.part_o + (row * p.splits + split) * HD + 4 * G;
+                float* o = p.part_o + (row * p.splits + split) * HDV + 4 * G;
 #pragma unroll
-                for (int db = 0; db < DB; ++db) *(f32x4*)(o + 16 * db) = acc[nb][db];
+                for (int db = 0; db < DBV; ++db) *(f32x4*)(o + 16 * db) = acc[nb][db];
                 if (G == 0) {
                     float* ml = p.part_ml + (row * p.splits + split) * 2;
                     ml[0] = m[nb];
@@ -1629,7 +1633,7 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         attn_decode_kernel<><<<fgrid, team * IA_WAVE, shared, stream>>>(p, fused->counters, team);
         IA_LAUNCH_CHECK("attention_decode");
         return 0;
-    } else if (HD == 128 && HDV == HD && g_tiles && cols >= 16 * TILE_NBW * TILE_WAVES && (splits == 1 || chunk % TILE_STAGE == 0)) {
+    } else if (TILE_FITS && g_tiles && cols >= 16 * TILE_NBW * TILE_WAVES && (splits == 1 || chunk % TILE_STAGE == 0)) {
         // portions of prompts: blocks of four waves that share the keys through shared memory
         // Blocks of 128 columns; of 64 (twice as many, the same bits) where the keys are not split and the blocks of 128
         // would be half a compute unit's worth or less, or, under a causal mask over most of the context, where the
@@ -1647,7 +1651,7 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         IA_CHECK(tiles <= 65535, "attention_mfma: %lld tiles of columns in a request (at most 65535)", tiles);
         const dim3 tgrid((unsigned)(nkv * splits * n_seqs), (unsigned)tiles, 1);
         p.pair = 0;
-        if (narrow) attn_tile_kernel<(HD == 128 && HDV == HD), 1><<<tgrid, TILE_GROUPS * TILE_WAVES * IA_WAVE, 0, stream>>>(p);
+        if (narrow) attn_tile_kernel<TILE_FITS, 1><<<tgrid, TILE_GROUPS * TILE_WAVES * IA_WAVE, 0, stream>>>(p);
         else attn_tile_kernel<><<<tgrid, TILE_GROUPS * TILE_WAVES * IA_WAVE, 0, stream>>>(p);
     } else if (nb == 1) {
         attn_mfma_kernel<1><<<grid, IA_WAVE, 0, stream>>>(p);

@@ -35,13 +35,14 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
 }
 
 #define IA_ROUTE_WAVES 4        // waves of a token's block
-#define IA_ROUTE_SHARE 8        // experts whose sums a wave holds at a time: a block takes 32 experts a round
+#define IA_ROUTE_SHARE 8        // experts whose sums a wave holds at a time: a block takes 32 experts a round (routers of 33 to 64
+                                // outputs: 10, 12 or 16, so that one walk over the row serves them all)
 
 // The logits: a block of four waves a token; in every round of 32 experts a wave takes eight.  A lane owns the features
 // 8 lane + 512 i of the row and adds its products up in that order (32-bit multiply-adds), then the lanes' sums meet in a
 // butterfly: an order that depends on the width alone.  The logits meet in shared memory and the first wave picks.
 // VEC: the width is a multiple of 8 (16-byte loads); else element by element.
-template <typename T, bool VEC>
+template <typename T, bool VEC, int SHARE = IA_ROUTE_SHARE>
 __global__ __launch_bounds__(64 * IA_ROUTE_WAVES) void route_kernel(int* __restrict__ sel, float* __restrict__ weight,
                                                                     const T* __restrict__ h, const T* __restrict__ wr, int n,
                                                                     int W, int E, int top, float scale, int score_fn,
@@ -49,10 +50,10 @@ __global__ __launch_bounds__(64 * IA_ROUTE_WAVES) void route_kernel(int* __restr
     __shared__ float logits[IA_MAX_EXPERTS];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const T* row = h + (long long)t * W;
-    for (int e0 = wave * IA_ROUTE_SHARE; e0 < E; e0 += IA_ROUTE_WAVES * IA_ROUTE_SHARE) {
-        float acc[IA_ROUTE_SHARE];
+    for (int e0 = wave * SHARE; e0 < E; e0 += IA_ROUTE_WAVES * SHARE) {
+        float acc[SHARE];
 #pragma unroll
-        for (int j = 0; j < IA_ROUTE_SHARE; ++j) acc[j] = 0.f;
+        for (int j = 0; j < SHARE; ++j) acc[j] = 0.f;
         // (four rounds of loads under way at once: a round is a trip to the memory)
 #pragma unroll 4
         for (int c0 = lane * 8; c0 < W; c0 += IA_WAVE * 8) {
@@ -64,7 +65,7 @@ __global__ __launch_bounds__(64 * IA_ROUTE_WAVES) void route_kernel(int* __restr
                 for (int i = 0; i < 8; ++i) x[i] = c0 + i < W ? ld(row + c0 + i) : 0.f;
             }
 #pragma unroll
-            for (int j = 0; j < IA_ROUTE_SHARE; ++j) {
+            for (int j = 0; j < SHARE; ++j) {
                 // (an expert beyond the last reads the last one's row: no branch stands between the loads)
                 const T* w = wr + (long long)(e0 + j < E ? e0 + j : E - 1) * W + c0;
                 float wv[8];
@@ -79,7 +80,7 @@ __global__ __launch_bounds__(64 * IA_ROUTE_WAVES) void route_kernel(int* __restr
             }
         }
 #pragma unroll
-        for (int j = 0; j < IA_ROUTE_SHARE; ++j) {
+        for (int j = 0; j < SHARE; ++j) {
             const float total = wave_sum(acc[j]);
             if (lane == 0 && e0 + j < E) logits[e0 + j] = total;
         }
@@ -332,9 +333,13 @@ extern "C" int ia_route(int* sel, float* weight, const void* h, const void* rout
     IA_CHECK(score_fn == IA_SCORE_SIGMOID || score_fn == IA_SCORE_SOFTMAX, "route: unknown score function %d", score_fn);
     if (n == 0) return 0;
     const bool vec = W % 8 == 0 && tile_mfma_aligned(h) && tile_mfma_aligned(router);
-#define IA_ROUTE(T, V) route_kernel<T, V><<<n, 64 * IA_ROUTE_WAVES, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm, choice_bias)
+#define IA_ROUTE_S(T, V, S) route_kernel<T, V, S><<<n, 64 * IA_ROUTE_WAVES, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm, choice_bias)
+    // (up to 32 outputs: 8 a wave; up to 64: as many a wave as take them all in one walk over the row)
+#define IA_ROUTE(T, V) do { if (E <= 32 || E > 64) IA_ROUTE_S(T, V, 8); else if (E <= 40) IA_ROUTE_S(T, V, 10); \
+        else if (E <= 48) IA_ROUTE_S(T, V, 12); else IA_ROUTE_S(T, V, 16); } while (0)
     if (dtype == IA_F32) { if (vec) IA_ROUTE(float, true); else IA_ROUTE(float, false); }
     else { if (vec) IA_ROUTE(bf16_t, true); else IA_ROUTE(bf16_t, false); }
+#undef IA_ROUTE_S
 #undef IA_ROUTE
     IA_LAUNCH_CHECK("route");
     return 0;

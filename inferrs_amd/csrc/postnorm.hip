@@ -54,6 +54,101 @@ __global__ __launch_bounds__(1024) void postnorm_step_kernel(
     }
 }
 
+// The same for widths in steps of 8 up to 8 * PN_VEC_ITERS * the block's threads: a thread owns eight neighbouring
+// features a round (16- and 32-byte accesses), the row's sum stays in its registers between the two passes, and nothing
+// goes through shared memory but the sum of squares.  The arithmetic of a feature is that of the kernel above.
+#define PN_VEC_ITERS 4
+
+__device__ __forceinline__ void pn_load8(const float* p, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void pn_load8(const bf16_t* p, float (&v)[8]) {
+    const uint4 a = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+__device__ __forceinline__ void pn_store8(float* p, const float (&v)[8]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void pn_store8(bf16_t* p, const float (&v)[8]) {
+    *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]),
+                                              pack_bf16x2(v[6], v[7]));
+}
+
+template <typename TY, typename TH>
+__global__ __launch_bounds__(1024) void postnorm_step_vec_kernel(
+    float* __restrict__ x, float alpha, const TY* __restrict__ y, const TY* __restrict__ y2,
+    const float* __restrict__ routed, const float* __restrict__ routed_w, const int* __restrict__ sel, int top,
+    int real_experts, const float* __restrict__ w, float eps, TH* __restrict__ h, const int* __restrict__ rows, int W) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int row = rows != nullptr ? rows[r] : r;
+    float* xr = x + (long long)row * W;
+    float wk[PN_MAX_TOP];
+    bool own[PN_MAX_TOP];
+#pragma unroll
+    for (int k = 0; k < PN_MAX_TOP; ++k) {
+        const bool on = routed != nullptr && k < top;
+        wk[k] = on ? routed_w[(long long)row * top + k] : 0.f;
+        own[k] = on && sel != nullptr && sel[(long long)row * top + k] >= real_experts;
+    }
+    float v[PN_VEC_ITERS][8];
+    float sq = 0.f;
+#pragma unroll
+    for (int it = 0; it < PN_VEC_ITERS; ++it) {
+        const int c = (it * blockDim.x + threadIdx.x) * 8;
+        if (c >= W) continue;
+        float xv[8], t[8];
+        pn_load8(xr + c, xv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[it][i] = alpha * xv[i];
+        if (y != nullptr) {
+            pn_load8(y + (long long)row * W + c, t);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[it][i] += t[i];
+        }
+        if (routed != nullptr) {
+#pragma unroll
+            for (int k = 0; k < PN_MAX_TOP; ++k) {
+                if (k >= top) break;
+                if (own[k]) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[it][i] = fmaf(wk[k], xv[i], v[it][i]);
+                } else {
+                    pn_load8(routed + ((long long)row * top + k) * W + c, t);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[it][i] = fmaf(wk[k], t[i], v[it][i]);
+                }
+            }
+        }
+        if (y2 != nullptr) {
+            pn_load8(y2 + (long long)row * W + c, t);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[it][i] += t[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sq = fmaf(v[it][i], v[it][i], sq);
+    }
+    const float rs = 1.0f / sqrtf(block_sum(sq, scratch) / (float)W + eps);
+#pragma unroll
+    for (int it = 0; it < PN_VEC_ITERS; ++it) {
+        const int c = (it * blockDim.x + threadIdx.x) * 8;
+        if (c >= W) continue;
+        float wv[8], o[8];
+        pn_load8(w + c, wv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = v[it][i] * rs * wv[i];
+        if (rows == nullptr) pn_store8(xr + c, o);
+        if (h != nullptr) pn_store8(h + (long long)r * W + c, o);
+    }
+}
+
 // y_dtype: precision of y and y2; h_dtype: of h.  0 float32, 1 bfloat16.
 extern "C" int ia_postnorm_step(float* x, float alpha, const void* y, const void* y2, const float* routed,
                                 const float* routed_w, const int* sel, int top, int real_experts, const float* w, float eps,
@@ -64,6 +159,23 @@ extern "C" int ia_postnorm_step(float* x, float alpha, const void* y, const void
              "postnorm_step: routed rows come with their weights, up to %d a row (top=%d)", PN_MAX_TOP, top);
     IA_CHECK(rows == nullptr || h != nullptr, "postnorm_step: a row list leaves the stream alone, so it needs an output");
     if (n == 0) return 0;
+    const uintptr_t ptrs = (uintptr_t)x | (uintptr_t)y | (uintptr_t)y2 | (uintptr_t)routed | (uintptr_t)w | (uintptr_t)h;
+    if (W % 8 == 0 && (ptrs & 15) == 0 && W <= 8 * PN_VEC_ITERS * 1024) {
+        // as many threads as the row has pieces of eight, in whole waves, a round or more each
+        int threads = (W / 8 + 63) / 64 * 64;
+        if (threads > 256) threads = (W / 8 + 2 * 64 - 1) / (2 * 64) * 64;          // two rounds a thread
+        if (threads > 512) threads = (W / 8 + PN_VEC_ITERS * 64 - 1) / (PN_VEC_ITERS * 64) * 64;
+#define IA_LAUNCH_VEC(TY, TH)                                                                                          \
+    postnorm_step_vec_kernel<TY, TH><<<n, threads, 0, stream>>>(x, alpha, (const TY*)y, (const TY*)y2, routed, routed_w, \
+                                                                sel, top, real_experts, w, eps, (TH*)h, rows, W)
+        if (y_dtype == IA_F32 && h_dtype == IA_F32) { IA_LAUNCH_VEC(float, float); }
+        else if (y_dtype == IA_F32) { IA_LAUNCH_VEC(float, bf16_t); }
+        else if (h_dtype == IA_F32) { IA_LAUNCH_VEC(bf16_t, float); }
+        else { IA_LAUNCH_VEC(bf16_t, bf16_t); }
+#undef IA_LAUNCH_VEC
+        IA_LAUNCH_CHECK("postnorm_step");
+        return 0;
+    }
     const int threads = W >= 4096 ? 1024 : W >= 1024 ? 512 : 256;
     const size_t shm = (size_t)W * sizeof(float);
 #define IA_LAUNCH(TY, TH)                                                                                            \

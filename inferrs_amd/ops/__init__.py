@@ -536,8 +536,10 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     elif tuple(out.shape) != (n, nq, dv) or out.dtype != q.dtype:
         raise KernelError("attention_mfma: `out` must be [n, nq, the values' width] in the dtype of q")
     if splits is None:
-        # (values of a width of their own stay on the kernel of single waves: its rule for splitting the keys)
-        splits, chunk = attention_split(n_seqs, nkv, nq // nkv, max_q_len, max_kv_len, d if dv == d else 0)
+        # (keys of 128 with values of 32 to 128 in steps of 32 have the kernel of blocks that share a stage, and its rule
+        # for splitting the keys; other pairs of widths stay on the kernel of single waves)
+        tiles = d == 128 and dv % 32 == 0 and dv <= 128
+        splits, chunk = attention_split(n_seqs, nkv, nq // nkv, max_q_len, max_kv_len, d if tiles or dv == d else 0)
     else:
         chunk = -(-(-(-max_kv_len // splits)) // 64) * 64
     target = _build.attn_target(d, dv)

@@ -303,7 +303,7 @@ def test_attention_generic_in_segments_is_the_same_bits_as_in_one_walk(dtype, nq
     bound = ops.attention_generic(*args, window=window, scale=scale, split=True, max_kv_len=max(lens))
     assert torch.equal(whole, parts) and torch.equal(whole, bound)
     close(whole, want, tol(dtype, 5e-6, 2 ** -7), "attention in segments")
-    assert ops.library().ia_attention_generic_workspace(4096, nq, nkv, d, 2000) == 0          # tokens enough: no split
+    assert ops.library().ia_attention_generic_workspace(4096, nq, nkv, d, d, 2000) == 0          # tokens enough: no split
     with pytest.raises(ops.KernelError):
         ops.attention_generic(*args, window=window, scale=scale, split=True, max_kv_len=300)  # one segment: nothing to split
 
