@@ -174,7 +174,8 @@ class FisanexConfig:
             names = (p + "norm1",) + ((p + "norm2",) if ffn is not None else ())
             layers.append(LayerSpec(mixer=self._mixer(i, layer, hidden, eps, sources), ffn=ffn, norms=(norm,) * len(names),
                                     norm_names=names, mixer_prefix=p + "mix.", ffn_prefix=p + "mlp.",
-                                    arrangement="post_norm", residual=PostNormSpec(alpha)))
+                                    arrangement="post_norm",
+                                    residual=PostNormSpec(alpha, bare_norm_name=None if ffn is not None else p + "norm2")))
         max_position = int(raw.get("max_position") or DEFAULT_MAX_POSITION)
         return ModelSpec(
             architecture=self.architecture, vocab_size=vocab, hidden=hidden, layers=tuple(layers),

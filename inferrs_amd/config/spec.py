@@ -258,8 +258,11 @@ class ClampedMlpSpec:
 @dataclass(frozen=True)
 class PostNormSpec:
     """How a layer's sub-layers stand around a stream that is normed after every sum (kept in 32-bit):
-    x <- norm(alpha x + part(x)), the parts reading x as it stands."""
+    x <- norm(alpha x + part(x)), the parts reading x as it stands.  `bare_norm_name`: a layer without a feed-forward
+    whose file still holds a second norm under this name runs it on the scaled stream alone, x <- norm(alpha x); a file
+    without the tensor leaves the step out."""
     alpha: float = 1.0
+    bare_norm_name: Optional[str] = None
 
 
 @dataclass(frozen=True)

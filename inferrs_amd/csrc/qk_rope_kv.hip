@@ -162,6 +162,106 @@ __global__ __launch_bounds__(QK_WAVES * IA_WAVE) void qk_rope_kv_strided_kernel(
     for (int j = rot + lane; j < d; j += IA_WAVE) st(dst + j, row[j]);
 }
 
+// The same with 16-byte accesses, for bfloat16 rows whose head sizes, pitch and offsets are multiples of 8: a thread owns
+// eight neighbouring features of one (token, head); the threads of a head meet in shared memory for the sum of squares
+// (added up in the order of the features) and for their rotation partners.  The blocks from `qk_blocks` on take the
+// values, eight features of a (token, key/value head) a thread, which go to their page slot by slot.
+#define QKS_THREADS 256
+__global__ __launch_bounds__(QKS_THREADS) void qk_rope_kv_strided_bf16_vec_kernel(
+    bf16_t* __restrict__ q_out, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, const bf16_t* __restrict__ proj,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, const int* __restrict__ slots, int n, int ld_, int q_off, int k_off, int v_off, int nq,
+    int nkv, int d, int dv, int rot, int interleaved, int page_size, float eps, int add_one, int qk_blocks) {
+    __shared__ float rows[QKS_THREADS * 8];          // normalised features, unit after unit
+    __shared__ float partial[QKS_THREADS];
+    if ((int)blockIdx.x >= qk_blocks) {
+        const int tpu = dv / 8, upb = QKS_THREADS / tpu;
+        const int u = threadIdx.x / tpu, t = threadIdx.x - u * tpu;
+        const long long unit = (long long)((int)blockIdx.x - qk_blocks) * upb + u;
+        if (u >= upb || unit >= (long long)n * nkv) return;
+        const int tok = (int)(unit / nkv), hh = (int)(unit % nkv);
+        const uint4 v = *(const uint4*)(proj + (size_t)tok * ld_ + v_off + hh * dv + t * 8);
+        const int slot = slots[tok];
+        const int page = slot / page_size, off = slot - page * page_size;
+        bf16_t* dst = v_cache + (((size_t)page * nkv + hh) * dv + t * 8) * page_size + off;
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[(size_t)j * page_size].bits = (uint16_t)(j & 1 ? w[j >> 1] >> 16 : w[j >> 1] & 0xffffu);
+        return;
+    }
+    const int tpu = d / 8, upb = QKS_THREADS / tpu;
+    const int u = threadIdx.x / tpu, t = threadIdx.x - u * tpu;
+    const int heads = slots ? nq + nkv : nq;
+    const long long unit = (long long)blockIdx.x * upb + u;
+    const bool active = u < upb && unit < (long long)n * heads;
+    const int tok = active ? (int)(unit / heads) : 0;
+    const int hh = active ? (int)(unit % heads) : 0;
+    const bool is_q = hh < nq;
+    const float* nw = is_q ? q_norm_w : k_norm_w;
+    float v[8];
+    float ss = 0.f;
+    if (active) {
+        const uint4 raw = *(const uint4*)(proj + (size_t)tok * ld_ + (is_q ? q_off + hh * d : k_off + (hh - nq) * d) + t * 8);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[2 * j] = __uint_as_float(w[j] << 16);
+            v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss = fmaf(v[j], v[j], ss);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = 0.f;
+    }
+    if (q_norm_w != nullptr || k_norm_w != nullptr) {                    // (the same for all threads: they meet at the barrier)
+        partial[threadIdx.x] = ss;
+        __syncthreads();
+        float total = 0.f;
+        if (active)
+            for (int j = 0; j < tpu; ++j) total += partial[u * tpu + j];
+        const float scale = 1.0f / sqrtf(total / (float)d + eps);
+        if (active && nw != nullptr) {
+            const float4 g0 = *(const float4*)(nw + t * 8), g1 = *(const float4*)(nw + t * 8 + 4);
+            const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = scale * v[j] * (add_one ? 1.0f + g[j] : g[j]);
+        }
+    }
+    const bool rotates = cos_t != nullptr && t * 8 < rot;               // (the same for all threads up to the barrier below)
+    if (cos_t != nullptr) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) rows[threadIdx.x * 8 + j] = v[j];
+        __syncthreads();
+    }
+    if (!active) return;
+    float o[8];
+    const int half = rot / 2;
+    const float* mine = rows + (size_t)u * tpu * 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int e = t * 8 + j;
+        o[j] = v[j];
+        if (rotates && e < rot) {
+            const bool first = interleaved ? (e & 1) == 0 : e < half;
+            const int i = interleaved ? e >> 1 : (first ? e : e - half);
+            const int other = interleaved ? e ^ 1 : (first ? e + half : e - half);
+            const float c = cos_t[(size_t)tok * half + i], sn = sin_t[(size_t)tok * half + i];
+            const float partner = mine[other];
+            o[j] = first ? v[j] * c - partner * sn : partner * sn + v[j] * c;
+        }
+    }
+    bf16_t* dst;
+    if (is_q) {
+        dst = q_out + ((size_t)tok * nq + hh) * d + t * 8;
+    } else {
+        const int slot = slots[tok];
+        const int page = slot / page_size, off = slot - page * page_size;
+        dst = k_cache + (((size_t)page * nkv + (hh - nq)) * page_size + off) * d + t * 8;
+    }
+    *(uint4*)dst = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+}
+
 extern "C" int ia_qk_rope_kv_strided(void* q_out, void* k_cache, void* v_cache, const void* proj, const float* q_norm_w,
                                      const float* k_norm_w, const float* cos_t, const float* sin_t, const int* slots, int n,
                                      int ld_, int q_off, int k_off, int v_off, int nq, int nkv, int d, int dv, int rot,
@@ -179,6 +279,21 @@ extern "C" int ia_qk_rope_kv_strided(void* q_out, void* k_cache, void* v_cache, 
     if (n == 0) return 0;
     const long long units = (long long)n * (slots ? nq + 2 * nkv : nq);
     const unsigned grid = (unsigned)((units + QK_WAVES - 1) / QK_WAVES);
+    const uintptr_t ptrs = (uintptr_t)q_out | (uintptr_t)proj | (uintptr_t)(slots ? k_cache : nullptr) | (uintptr_t)q_norm_w |
+                           (uintptr_t)k_norm_w;
+    if (dtype == IA_BF16 && d % 8 == 0 && dv % 8 == 0 && d / 8 <= QKS_THREADS && dv / 8 <= QKS_THREADS && ld_ % 8 == 0 &&
+        q_off % 8 == 0 && (slots == nullptr || (k_off % 8 == 0 && v_off % 8 == 0)) && (ptrs & 15) == 0) {
+        const long long qk_units = (long long)n * (slots ? nq + nkv : nq);
+        const int upb = QKS_THREADS / (d / 8), upb_v = QKS_THREADS / (dv / 8);
+        const long long qk_blocks = (qk_units + upb - 1) / upb;
+        const long long v_blocks = slots ? ((long long)n * nkv + upb_v - 1) / upb_v : 0;
+        IA_CHECK(qk_blocks + v_blocks < (1ll << 31), "qk_rope_kv_strided: %d tokens are too many for one launch", n);
+        qk_rope_kv_strided_bf16_vec_kernel<<<(unsigned)(qk_blocks + v_blocks), QKS_THREADS, 0, stream>>>(
+            (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, (const bf16_t*)proj, q_norm_w, k_norm_w, cos_t, sin_t, slots, n,
+            ld_, q_off, k_off, v_off, nq, nkv, d, dv, rot, interleaved, page_size, eps, add_one, (int)qk_blocks);
+        IA_LAUNCH_CHECK("qk_rope_kv_strided");
+        return 0;
+    }
     if (dtype == IA_F32)
         qk_rope_kv_strided_kernel<float><<<grid, QK_WAVES * IA_WAVE, 0, stream>>>(
             (float*)q_out, (float*)k_cache, (float*)v_cache, (const float*)proj, q_norm_w, k_norm_w, cos_t, sin_t, slots, n,

@@ -25,6 +25,10 @@ def model_tensors(spec: ModelSpec) -> Tuple[Dict[str, TensorSpec], Set[str]]:
     if getattr(spec, "pass_input", None) is not None:
         expected.update(part_class("pass_input", spec.pass_input).tensors(spec.pass_input))
     optional: Set[str] = set(head.optional(spec.head)) if hasattr(head, "optional") else set()
+    for layer in spec.layers:                    # (a block arrangement may name tensors that a file may leave out)
+        cls = block_class(layer)
+        if hasattr(cls, "optional"):
+            optional |= set(cls.optional(layer))
     return expected, optional
 
 

@@ -42,7 +42,16 @@ class PostNormBlock(BlockBase):
         for name, nspec in zip(spec.norm_names, spec.norms):
             (ts,) = part_class("norm", nspec).tensors(nspec).values()
             out[name] = ts
+        for name in cls.optional(spec):
+            (ts,) = part_class("norm", spec.norms[0]).tensors(spec.norms[0]).values()
+            out[name] = ts
         return out
+
+    @classmethod
+    def optional(cls, spec: LayerSpec):
+        """Names that a file may leave out: the second norm of a layer that has no feed-forward."""
+        name = getattr(spec.residual, "bare_norm_name", None)
+        return {name} if spec.ffn is None and name else set()
 
     def __init__(self, spec: LayerSpec, tensors: Dict[str, torch.Tensor], dtype, device):
         self.spec, self.dtype = spec, dtype
@@ -58,6 +67,9 @@ class PostNormBlock(BlockBase):
                       for name, nspec in zip(spec.norm_names, spec.norms)]
         if len(self.norms) != (1 if self.ffn is None else 2):
             raise SpecError("post_norm: a norm behind every sub-layer")
+        for name in self.optional(spec):
+            if name in tensors:                 # (the file holds a second norm for a layer without a feed-forward)
+                self.norms.append(part_class("norm", spec.norms[0])(spec.norms[0], {"weight": tensors[name]}, dtype, device))
         for n in self.norms:
             if getattr(n, "add_one", False) or not hasattr(n, "weight") or not hasattr(n, "eps"):
                 raise SpecError("post_norm: the norms must be plain RMS norms")
@@ -89,8 +101,12 @@ class PostNormBlock(BlockBase):
     # ---- a layer ------------------------------------------------------------------------------------
     def _close(self, x: torch.Tensor, out, norm):
         """x <- norm(alpha x + out); returns what the next products read."""
-        extra = dict(routed=out.rows, routed_weights=out.weights, sel=out.sel, real_experts=out.real_experts,
-                     y2=out.extra) if isinstance(out, RoutedRows) else dict(y=out.materialize() if hasattr(out, "materialize") else out)
+        if out is None:
+            extra = {}
+        elif isinstance(out, RoutedRows):
+            extra = dict(routed=out.rows, routed_weights=out.weights, sel=out.sel, real_experts=out.real_experts, y2=out.extra)
+        else:
+            extra = dict(y=out.materialize() if hasattr(out, "materialize") else out)
         h = ops.postnorm_step(x, alpha=self.alpha, weight=norm.weight, eps=norm.eps,
                               h_dtype=None if self.dtype == torch.float32 else self.dtype, **extra)
         return x if h is None else h
@@ -108,5 +124,7 @@ class PostNormBlock(BlockBase):
         h = self._close(x, self.mixer.forward(ctx, h, cache), self.norms[0])
         if self.ffn is not None:
             h = self._close(x, self.ffn.forward(ctx, h), self.norms[1])
+        elif len(self.norms) > 1:
+            h = self._close(x, None, self.norms[1])
         ctx.post_rows = h
         return x, None

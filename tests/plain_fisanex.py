@@ -141,6 +141,8 @@ def forward(cfg: dict, w: T, tokens: Sequence[int], dtype=torch.float64, layers_
         x = rms_norm(alpha * x + windowed_attention(x, w, p + "mix.", m, eps, k, v), w[p + "norm1"], eps)
         if layer.get("mlp") is not None:
             x = rms_norm(alpha * x + feed_forward(x, w, p + "mlp.", layer["mlp"]), w[p + "norm2"], eps)
+        elif p + "norm2" in w:                  # (a file that holds a second norm for a layer without a feed-forward)
+            x = rms_norm(alpha * x, w[p + "norm2"], eps)
         if layers_out is not None:
             layers_out.append(x.clone())
     x = rms_norm(x, w["final.norm"], eps)

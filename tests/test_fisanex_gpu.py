@@ -456,6 +456,27 @@ def test_decode_steps_replayed_from_graphs(models):
         assert err <= 3e-2, (graphs, err)
 
 
+def test_a_second_norm_without_a_feed_forward(models, tmp_path):
+    """A file that holds a second norm for a layer without a feed-forward: the scaled stream goes through it."""
+    from inferrs_amd.engine import Engine
+    from inferrs_amd.engine.engine import Entry
+    from inferrs_amd.weights import write_safetensors
+    folder, cfg, tensors, reqs, ref = models[("A", 1.0)]
+    more = dict(tensors, **{"l3.norm2": (0.5 + torch.rand(cfg["width"])).to(torch.bfloat16)})
+    new = str(tmp_path / "with_norm2")
+    os.makedirs(new)
+    with open(os.path.join(new, "config.json"), "w") as f:
+        import json
+        json.dump(cfg, f)
+    write_safetensors(os.path.join(new, "model.safetensors"), more)
+    toks = reqs["r5"]
+    want = pf.forward(cfg, more, toks)
+    assert float((want - torch.from_numpy(ref["r5"]).double()).abs().max()) > 1e-2
+    eng = Engine.from_folder(new, dtype="float32", page_size=16, num_pages=8, max_seqs=2)
+    got = eng.step([Entry("a", toks, list(range(len(toks))))]).double().cpu()
+    assert float((got - want).abs().max()) <= TOL_F32 * float(want.abs().max())
+
+
 def test_random_weights_engine_steps():
     """The measurement script's way in: a configuration object and weights drawn on the device."""
     from inferrs_amd.config.fisanex import FisanexConfig
