@@ -213,7 +213,8 @@ int ia_activation(void* x, long long n, int act, int dtype, hipStream_t stream);
 // routed[k] + y2) * w, written back in 32-bit and to h (h_dtype; null: not wanted); every addend may be null.  routed
 // [n, top, W] 32-bit with weights [n, top]; a pair whose sel (null: none) is real_experts or more stands for the stream's
 // own row.  rows: only these rows are read, the stream is left alone and h gets one row for each.
-int ia_postnorm_step(float* x, float alpha, const void* y, const void* y2, const float* routed,
+// y_splits, y2_splits: 1, or y (y2) is a 32-bit product still split along its k, [splits, n, W], added up here.
+int ia_postnorm_step(float* x, float alpha, const void* y, const void* y2, int y_splits, int y2_splits, const float* routed,
                      const float* routed_w, const int* sel, int top, int real_experts, const float* w, float eps,
                      void* h, const int* rows, int n, int W, int y_dtype, int h_dtype, hipStream_t stream);
 // out (32-bit) = table[ids] * scale; h (null: not wanted): the same rows in the table's precision

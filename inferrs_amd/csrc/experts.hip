@@ -35,6 +35,7 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
 }
 
 #define IA_ROUTE_WAVES 4        // waves of a token's block
+#define IA_ROUTE_FEW_TOKENS 64 // up to this many tokens a step the blocks are too few to hide a wave's chain of loads
 #define IA_ROUTE_SHARE 8        // experts whose sums a wave holds at a time: a block takes 32 experts a round (routers of 33 to 64
                                 // outputs: 10, 12 or 16, so that one walk over the row serves them all)
 
@@ -42,15 +43,16 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
 // 8 lane + 512 i of the row and adds its products up in that order (32-bit multiply-adds), then the lanes' sums meet in a
 // butterfly: an order that depends on the width alone.  The logits meet in shared memory and the first wave picks.
 // VEC: the width is a multiple of 8 (16-byte loads); else element by element.
-template <typename T, bool VEC, int SHARE = IA_ROUTE_SHARE>
-__global__ __launch_bounds__(64 * IA_ROUTE_WAVES) void route_kernel(int* __restrict__ sel, float* __restrict__ weight,
+// WAVES: the block's waves.  A logit is one wave's walk over the row whatever SHARE and WAVES are, so neither changes a sum.
+template <typename T, bool VEC, int SHARE = IA_ROUTE_SHARE, int WAVES = IA_ROUTE_WAVES>
+__global__ __launch_bounds__(64 * WAVES) void route_kernel(int* __restrict__ sel, float* __restrict__ weight,
                                                                     const T* __restrict__ h, const T* __restrict__ wr, int n,
                                                                     int W, int E, int top, float scale, int score_fn,
                                                                     int renorm, const float* __restrict__ choice_bias) {
     __shared__ float logits[IA_MAX_EXPERTS];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const T* row = h + (long long)t * W;
-    for (int e0 = wave * SHARE; e0 < E; e0 += IA_ROUTE_WAVES * SHARE) {
+    for (int e0 = wave * SHARE; e0 < E; e0 += WAVES * SHARE) {
         float acc[SHARE];
 #pragma unroll
         for (int j = 0; j < SHARE; ++j) acc[j] = 0.f;
@@ -333,12 +335,19 @@ extern "C" int ia_route(int* sel, float* weight, const void* h, const void* rout
     IA_CHECK(score_fn == IA_SCORE_SIGMOID || score_fn == IA_SCORE_SOFTMAX, "route: unknown score function %d", score_fn);
     if (n == 0) return 0;
     const bool vec = W % 8 == 0 && tile_mfma_aligned(h) && tile_mfma_aligned(router);
-#define IA_ROUTE_S(T, V, S) route_kernel<T, V, S><<<n, 64 * IA_ROUTE_WAVES, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm, choice_bias)
-    // (up to 32 outputs: 8 a wave; up to 64: as many a wave as take them all in one walk over the row)
-#define IA_ROUTE(T, V) do { if (E <= 32 || E > 64) IA_ROUTE_S(T, V, 8); else if (E <= 40) IA_ROUTE_S(T, V, 10); \
+#define IA_ROUTE_SW(T, V, S, WV) route_kernel<T, V, S, WV><<<n, 64 * WV, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm, choice_bias)
+#define IA_ROUTE_S(T, V, S) IA_ROUTE_SW(T, V, S, IA_ROUTE_WAVES)
+    // (up to 32 outputs: 8 a wave; up to 64: as many a wave as take them all in one walk over the row.  A step of few
+    // tokens has few blocks, and a wave's walk is a chain of trips to the memory: sixteen waves a token then, each with
+    // as few outputs as share them all out)
+#define IA_ROUTE(T, V) do { if (n <= IA_ROUTE_FEW_TOKENS && E > 8) { \
+            if (E <= 16) IA_ROUTE_SW(T, V, 1, 16); else if (E <= 32) IA_ROUTE_SW(T, V, 2, 16); \
+            else if (E <= 48) IA_ROUTE_SW(T, V, 3, 16); else if (E <= 64) IA_ROUTE_SW(T, V, 4, 16); else IA_ROUTE_SW(T, V, 8, 16); } \
+        else if (E <= 32 || E > 64) IA_ROUTE_S(T, V, 8); else if (E <= 40) IA_ROUTE_S(T, V, 10); \
         else if (E <= 48) IA_ROUTE_S(T, V, 12); else IA_ROUTE_S(T, V, 16); } while (0)
     if (dtype == IA_F32) { if (vec) IA_ROUTE(float, true); else IA_ROUTE(float, false); }
     else { if (vec) IA_ROUTE(bf16_t, true); else IA_ROUTE(bf16_t, false); }
+#undef IA_ROUTE_SW
 #undef IA_ROUTE_S
 #undef IA_ROUTE
     IA_LAUNCH_CHECK("route");

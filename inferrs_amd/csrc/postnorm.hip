@@ -14,11 +14,20 @@
 
 #define PN_MAX_TOP 16
 
+// An output that is still split along the k of its product, [splits, n, W]: the splits' sums added up in their order.
+template <typename T>
+__device__ __forceinline__ float pn_sum_splits(const T* p, int splits, long long stride) {
+    float t = ld(p);
+    for (int s = 1; s < splits; ++s) t += ld(p + s * stride);
+    return t;
+}
+
 template <typename TY, typename TH>
 __global__ __launch_bounds__(1024) void postnorm_step_kernel(
-    float* __restrict__ x, float alpha, const TY* __restrict__ y, const TY* __restrict__ y2,
-    const float* __restrict__ routed, const float* __restrict__ routed_w, const int* __restrict__ sel, int top,
-    int real_experts, const float* __restrict__ w, float eps, TH* __restrict__ h, const int* __restrict__ rows, int W) {
+    float* __restrict__ x, float alpha, const TY* __restrict__ y, const TY* __restrict__ y2, int y_splits, int y2_splits,
+    long long split_stride, const float* __restrict__ routed, const float* __restrict__ routed_w,
+    const int* __restrict__ sel, int top, int real_experts, const float* __restrict__ w, float eps, TH* __restrict__ h,
+    const int* __restrict__ rows, int W) {
     extern __shared__ float pn_row[];            // [W]
     __shared__ float scratch[16];
     const int r = blockIdx.x;
@@ -36,13 +45,13 @@ __global__ __launch_bounds__(1024) void postnorm_step_kernel(
     for (int c = threadIdx.x; c < W; c += blockDim.x) {
         const float xv = xr[c];
         float v = alpha * xv;
-        if (y != nullptr) v += ld(y + (long long)row * W + c);
+        if (y != nullptr) v += pn_sum_splits(y + (long long)row * W + c, y_splits, split_stride);
         if (routed != nullptr) {
 #pragma unroll
             for (int k = 0; k < PN_MAX_TOP; ++k)
                 if (k < top) v = fmaf(wk[k], own[k] ? xv : routed[((long long)row * top + k) * W + c], v);
         }
-        if (y2 != nullptr) v += ld(y2 + (long long)row * W + c);
+        if (y2 != nullptr) v += pn_sum_splits(y2 + (long long)row * W + c, y2_splits, split_stride);
         pn_row[c] = v;
         sq = fmaf(v, v, sq);
     }
@@ -81,11 +90,23 @@ __device__ __forceinline__ void pn_store8(bf16_t* p, const float (&v)[8]) {
                                               pack_bf16x2(v[6], v[7]));
 }
 
+template <typename T>
+__device__ __forceinline__ void pn_load8_splits(const T* p, int splits, long long stride, float (&t)[8]) {
+    pn_load8(p, t);
+    for (int s = 1; s < splits; ++s) {
+        float u[8];
+        pn_load8(p + s * stride, u);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) t[i] += u[i];
+    }
+}
+
 template <typename TY, typename TH>
 __global__ __launch_bounds__(1024) void postnorm_step_vec_kernel(
-    float* __restrict__ x, float alpha, const TY* __restrict__ y, const TY* __restrict__ y2,
-    const float* __restrict__ routed, const float* __restrict__ routed_w, const int* __restrict__ sel, int top,
-    int real_experts, const float* __restrict__ w, float eps, TH* __restrict__ h, const int* __restrict__ rows, int W) {
+    float* __restrict__ x, float alpha, const TY* __restrict__ y, const TY* __restrict__ y2, int y_splits, int y2_splits,
+    long long split_stride, const float* __restrict__ routed, const float* __restrict__ routed_w,
+    const int* __restrict__ sel, int top, int real_experts, const float* __restrict__ w, float eps, TH* __restrict__ h,
+    const int* __restrict__ rows, int W) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int row = rows != nullptr ? rows[r] : r;
@@ -109,7 +130,7 @@ __global__ __launch_bounds__(1024) void postnorm_step_vec_kernel(
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[it][i] = alpha * xv[i];
         if (y != nullptr) {
-            pn_load8(y + (long long)row * W + c, t);
+            pn_load8_splits(y + (long long)row * W + c, y_splits, split_stride, t);
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[it][i] += t[i];
         }
@@ -128,7 +149,7 @@ __global__ __launch_bounds__(1024) void postnorm_step_vec_kernel(
             }
         }
         if (y2 != nullptr) {
-            pn_load8(y2 + (long long)row * W + c, t);
+            pn_load8_splits(y2 + (long long)row * W + c, y2_splits, split_stride, t);
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[it][i] += t[i];
         }
@@ -149,16 +170,21 @@ __global__ __launch_bounds__(1024) void postnorm_step_vec_kernel(
     }
 }
 
-// y_dtype: precision of y and y2; h_dtype: of h.  0 float32, 1 bfloat16.
-extern "C" int ia_postnorm_step(float* x, float alpha, const void* y, const void* y2, const float* routed,
-                                const float* routed_w, const int* sel, int top, int real_experts, const float* w, float eps,
-                                void* h, const int* rows, int n, int W, int y_dtype, int h_dtype, hipStream_t stream) {
+// y_dtype: precision of y and y2; h_dtype: of h.  0 float32, 1 bfloat16.  y_splits, y2_splits: 1, or the splits of a product
+// that is still split along its k ([splits, n, W], 32-bit), which the kernel adds up in their order.
+extern "C" int ia_postnorm_step(float* x, float alpha, const void* y, const void* y2, int y_splits, int y2_splits,
+                                const float* routed, const float* routed_w, const int* sel, int top, int real_experts,
+                                const float* w, float eps, void* h, const int* rows, int n, int W, int y_dtype, int h_dtype,
+                                hipStream_t stream) {
     IA_CHECK(n >= 0 && W > 0 && w != nullptr, "postnorm_step: n=%d width=%d, and the norm's weight", n, W);
     IA_CHECK((size_t)W * sizeof(float) <= 60 * 1024, "postnorm_step: width %d does not fit shared memory", W);
     IA_CHECK(routed == nullptr || (routed_w != nullptr && top >= 1 && top <= PN_MAX_TOP),
              "postnorm_step: routed rows come with their weights, up to %d a row (top=%d)", PN_MAX_TOP, top);
     IA_CHECK(rows == nullptr || h != nullptr, "postnorm_step: a row list leaves the stream alone, so it needs an output");
+    IA_CHECK(y_splits >= 1 && y2_splits >= 1 && ((y_splits == 1 && y2_splits == 1) || (y_dtype == IA_F32 && rows == nullptr)),
+             "postnorm_step: outputs in %d and %d splits are 32-bit and cover every row", y_splits, y2_splits);
     if (n == 0) return 0;
+    const long long split_stride = (long long)n * W;
     const uintptr_t ptrs = (uintptr_t)x | (uintptr_t)y | (uintptr_t)y2 | (uintptr_t)routed | (uintptr_t)w | (uintptr_t)h;
     if (W % 8 == 0 && (ptrs & 15) == 0 && W <= 8 * PN_VEC_ITERS * 1024) {
         // as many threads as the row has pieces of eight, in whole waves, a round or more each
@@ -166,8 +192,9 @@ extern "C" int ia_postnorm_step(float* x, float alpha, const void* y, const void
         if (threads > 256) threads = (W / 8 + 2 * 64 - 1) / (2 * 64) * 64;          // two rounds a thread
         if (threads > 512) threads = (W / 8 + PN_VEC_ITERS * 64 - 1) / (PN_VEC_ITERS * 64) * 64;
 #define IA_LAUNCH_VEC(TY, TH)                                                                                          \
-    postnorm_step_vec_kernel<TY, TH><<<n, threads, 0, stream>>>(x, alpha, (const TY*)y, (const TY*)y2, routed, routed_w, \
-                                                                sel, top, real_experts, w, eps, (TH*)h, rows, W)
+    postnorm_step_vec_kernel<TY, TH><<<n, threads, 0, stream>>>(x, alpha, (const TY*)y, (const TY*)y2, y_splits, y2_splits, \
+                                                                split_stride, routed, routed_w, sel, top, real_experts, w, eps, \
+                                                                (TH*)h, rows, W)
         if (y_dtype == IA_F32 && h_dtype == IA_F32) { IA_LAUNCH_VEC(float, float); }
         else if (y_dtype == IA_F32) { IA_LAUNCH_VEC(float, bf16_t); }
         else if (h_dtype == IA_F32) { IA_LAUNCH_VEC(bf16_t, float); }
@@ -179,8 +206,9 @@ extern "C" int ia_postnorm_step(float* x, float alpha, const void* y, const void
     const int threads = W >= 4096 ? 1024 : W >= 1024 ? 512 : 256;
     const size_t shm = (size_t)W * sizeof(float);
 #define IA_LAUNCH(TY, TH)                                                                                            \
-    postnorm_step_kernel<TY, TH><<<n, threads, shm, stream>>>(x, alpha, (const TY*)y, (const TY*)y2, routed, routed_w, \
-                                                              sel, top, real_experts, w, eps, (TH*)h, rows, W)
+    postnorm_step_kernel<TY, TH><<<n, threads, shm, stream>>>(x, alpha, (const TY*)y, (const TY*)y2, y_splits, y2_splits, \
+                                                              split_stride, routed, routed_w, sel, top, real_experts, w, eps, \
+                                                              (TH*)h, rows, W)
     if (y_dtype == IA_F32 && h_dtype == IA_F32) { IA_LAUNCH(float, float); }
     else if (y_dtype == IA_F32) { IA_LAUNCH(float, bf16_t); }
     else if (h_dtype == IA_F32) { IA_LAUNCH(bf16_t, float); }

@@ -296,16 +296,30 @@ def postnorm_step(x: torch.Tensor, *, alpha: float = 1.0, y: Optional[torch.Tens
 
         x <- rmsnorm(alpha x + y + sum_k routed_weights[:, k] * routed[:, k] + y2) * weight
 
-    and, with `h_dtype`, the new rows once more in that precision.  Every addend may be absent.  `routed` [n, top, width]
+    and, with `h_dtype`, the new rows once more in that precision.  Every addend may be absent.  y and y2 may each be a
+    product that is still split along its k (`Partials`, 32-bit [splits, n, width]): the kernel adds the splits up in
+    their order, nothing is rounded in between.  `routed` [n, top, width]
     (32-bit): with `sel` [n, top], a pair whose entry is `real_experts` or more stands for the stream's own row (an expert
     that hands its input on).  `rows` (int32): only these rows are read, the stream is left as it is and the result has one
     row for each of them."""
+    from . import Partials
+    both = [t for t in (y, y2) if t is not None]
+    if any(isinstance(t, Partials) for t in both) and any(not isinstance(t, Partials) and t.dtype != torch.float32 for t in both):
+        y, y2 = (t.materialize() if isinstance(t, Partials) else t for t in (y, y2))    # (one precision for both)
+    y_splits = y2_splits = 1
+    if isinstance(y, Partials):
+        y_splits, y = y.parts.shape[0], y.parts
+    if isinstance(y2, Partials):
+        y2_splits, y2 = y2.parts.shape[0], y2.parts
     _dev(x, y, y2, routed, routed_weights, sel, weight, rows)
     _f32(x, "the stream"); _f32(routed, "routed rows"); _f32(routed_weights, "routed weights"); _f32(weight, "norm weight")
     n, W = x.shape
     given = [t for t in (y, y2) if t is not None]
-    for t in given:
-        if tuple(t.shape) != (n, W) or t.dtype != given[0].dtype:
+    for t, splits in ((y, y_splits), (y2, y2_splits)):
+        if t is None:
+            continue
+        if (tuple(t.shape[-2:]) != (n, W) or t.dtype != given[0].dtype or not t.is_contiguous()
+                or (t.dim() == 3 and (t.shape[0] != splits or t.dtype != torch.float32)) or t.dim() not in (2, 3)):
             raise KernelError(f"postnorm_step: an output {tuple(t.shape)} {t.dtype} does not fit the stream [{n}, {W}]")
     top = 0
     if routed is not None:
@@ -327,7 +341,8 @@ def postnorm_step(x: torch.Tensor, *, alpha: float = 1.0, y: Optional[torch.Tens
             raise KernelError("postnorm_step: a row list goes with an output and nothing to add")
     h = torch.empty((count, W), dtype=h_dtype, device=x.device) if h_dtype is not None else None
     _check(library().ia_postnorm_step(
-        _p(x), ctypes.c_float(alpha), _p(y), _p(y2), _p(routed), _p(routed_weights), _p(sel), top, int(real_experts),
+        _p(x), ctypes.c_float(alpha), _p(y), _p(y2), y_splits, y2_splits, _p(routed), _p(routed_weights), _p(sel), top,
+        int(real_experts),
         _p(weight), ctypes.c_float(eps), _p(h), _p(rows), count, W, _dt(given[0]) if given else 0,
         _DT[h_dtype] if h_dtype is not None else 0, _stream()))
     return h

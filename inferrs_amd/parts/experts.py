@@ -122,4 +122,9 @@ class ClampedMlp(FeedForward):
     def forward(self, ctx, h):
         if hasattr(h, "materialize"):
             h = h.materialize()
-        return self.down(ops.clamped_gate_mul(self.gate_up(h), self.spec.limit, self.spec.alpha))
+        act = ops.clamped_gate_mul(self.gate_up(h), self.spec.limit, self.spec.alpha)
+        if getattr(ctx, "partial_sums", False):
+            split = ops.linear_partials(act, self.down.weight, self.down.bias)
+            if split is not None:
+                return split
+        return self.down(act)

@@ -106,7 +106,8 @@ class PostNormBlock(BlockBase):
         elif isinstance(out, RoutedRows):
             extra = dict(routed=out.rows, routed_weights=out.weights, sel=out.sel, real_experts=out.real_experts, y2=out.extra)
         else:
-            extra = dict(y=out.materialize() if hasattr(out, "materialize") else out)
+            # (a product still split along its k is added up by the kernel itself)
+            extra = dict(y=out if isinstance(out, ops.Partials) or not hasattr(out, "materialize") else out.materialize())
         h = ops.postnorm_step(x, alpha=self.alpha, weight=norm.weight, eps=norm.eps,
                               h_dtype=None if self.dtype == torch.float32 else self.dtype, **extra)
         return x if h is None else h
@@ -117,7 +118,8 @@ class PostNormBlock(BlockBase):
         if pending is not None:
             raise SpecError("post_norm: the block before leaves something that this arrangement does not take")
         ctx.stream = ctx.stream_norm = None
-        ctx.partial_sums = False
+        # steps of few rows: a part's last product may stay split along k (gemm_mid.hip), for `ops.postnorm_step` to add up
+        ctx.partial_sums = self.dtype == torch.bfloat16 and ops.MID_MIN_ROWS <= x.shape[0] <= ops.MID_MAX_ROWS
         h = getattr(ctx, "post_rows", None)
         if h is None or h.shape != x.shape:
             h = x if self.dtype == torch.float32 else x.to(self.dtype)
@@ -127,4 +129,5 @@ class PostNormBlock(BlockBase):
         elif len(self.norms) > 1:
             h = self._close(x, None, self.norms[1])
         ctx.post_rows = h
+        ctx.partial_sums = False
         return x, None

@@ -76,6 +76,19 @@ def test_step_behind_a_sublayer(W, y_dtype):
     rows = torch.where((sel >= real)[:, :, None], x.double()[:, None, :], routed.double().nan_to_num())
     want = pf.rms_norm(0.6 * x.double() + (rw.double()[:, :, None] * rows).sum(1) + y2.double(), w.double(), 1e-6)
     np.testing.assert_allclose(xs.cpu().numpy(), want.numpy(), rtol=1e-5, atol=1e-5)
+    # outputs that are products still split along their k: the kernel adds the splits up
+    if y_dtype == torch.float32:
+        parts, parts2 = (torch.randn(s, n, W, generator=g) for s in (3, 1))
+        xs2 = dev(x)
+        ops.postnorm_step(xs2, alpha=0.6, y=ops.Partials(dev(parts)), weight=dev(w), eps=1e-6)
+        np.testing.assert_allclose(xs2.cpu().numpy(), pf.rms_norm(0.6 * x.double() + parts.double().sum(0), w.double(), 1e-6).numpy(),
+                                   rtol=1e-5, atol=1e-5)
+        xs2 = dev(x)
+        ops.postnorm_step(xs2, alpha=0.6, routed=dev(routed), routed_weights=dev(rw), sel=dev(sel), real_experts=real,
+                          y=ops.Partials(dev(parts2)), y2=ops.Partials(dev(parts)), weight=dev(w), eps=1e-6)
+        want2 = pf.rms_norm(0.6 * x.double() + (rw.double()[:, :, None] * rows).sum(1) + parts.double().sum(0) + parts2.double().sum(0),
+                            w.double(), 1e-6)
+        np.testing.assert_allclose(xs2.cpu().numpy(), want2.numpy(), rtol=1e-5, atol=1e-5)
     # the model's end: some rows through a norm, the stream left as it is
     before = xs.clone()
     pick = torch.tensor([5, 0, 18], dtype=torch.int32)
