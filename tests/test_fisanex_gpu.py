@@ -285,6 +285,23 @@ def test_router_with_a_correction(E, identity, top, W, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("E,top,W", [(36, 4, 256), (12, 2, 50), (70, 6, 136), (200, 3, 64)])
+def test_router_does_not_depend_on_the_step(E, top, W, dtype):
+    """A step of few tokens and one of many launch the router differently (more waves a token, fewer outputs a wave): a
+    token's choice and weights are the same bits in both, wherever in a step the token stands."""
+    from inferrs_amd import ops
+    g = torch.Generator().manual_seed(E + W)
+    n = 1031
+    h = dev(torch.randn(n, W, generator=g).to(dtype))
+    router = dev((2 * torch.randn(E, W, generator=g) / W ** 0.5).to(dtype))
+    corr = dev(0.15 * torch.randn(E, generator=g))
+    sel, weight = ops.route(h, router, top, 1.0, "softmax", False, corr)
+    for first, count in ((0, 1), (3, 8), (40, 64), (100, 65), (500, 300), (1000, 31), (n - 1, 1)):
+        s2, w2 = ops.route(h[first:first + count].contiguous(), router, top, 1.0, "softmax", False, corr)
+        assert torch.equal(s2, sel[first:first + count]) and torch.equal(w2, weight[first:first + count]), (first, count)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("E,identity,top,W,ff", [(5, 2, 3, 48, 24), (3, 1, 2, 50, 30), (6, 3, 2, 64, 32)])
 def test_experts_leave_out_pairs_that_name_none(E, identity, top, W, ff, dtype):
     from inferrs_amd import ops
