@@ -70,10 +70,10 @@ CFG_C = model(101, 50, [
 # width of their own; long prompts, keys split between waves in decode steps), a window of 300 that two readers share, one
 # of them further down with a narrower window; values of 16 beside keys of 64 in the last layer.
 CFG_D = model(150, 64, [
-    layer(attn(4, 1, 128, 64, 0.09, 300, base=20000.0, turned=32), dense(48)),
+    layer(attn(4, 1, 128, 64, 0.09, 300, base=30000.0, turned=48), dense(48)),
     layer(attn(2, 2, 64, 16, 0.15, 64, base=100.0), None),
-    layer(attn(4, 1, 128, 64, 0.09, 300, base=20000.0, turned=32, kv_from=0), moe(6, 3, 2, 32, 1.5, shared=(16, 2.0))),
-    layer(attn(4, 1, 128, 64, 0.12, 33, base=20000.0, turned=32, kv_from=0), dense(48))],
+    layer(attn(4, 1, 128, 64, 0.09, 300, base=30000.0, turned=48, kv_from=0), moe(6, 3, 2, 32, 1.3, shared=(16, 2.2))),
+    layer(attn(4, 1, 128, 64, 0.12, 33, base=30000.0, turned=48, kv_from=0), dense(48))],
     alpha=2.5, embed_scale=8.0, logit_scale=0.3)
 CONFIGS = {"A": CFG_A, "B": CFG_B, "C": CFG_C, "D": CFG_D}
 
