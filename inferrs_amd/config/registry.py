@@ -20,6 +20,7 @@ from typing import Any, Dict, Optional, Type
 from .base import ConfigError, read_config_json
 from .buketar import BuketarConfig
 from .fisanex import FisanexConfig
+from .ligizen import LigizenConfig
 from .lofudra import LofudraConfig
 from .qwen3 import Qwen3Config
 from .spec import ModelSpec
@@ -74,3 +75,4 @@ register_architecture(Qwen3Config)
 register_architecture(BuketarConfig)
 register_architecture(LofudraConfig)
 register_architecture(FisanexConfig)
+register_architecture(LigizenConfig)

@@ -31,6 +31,16 @@ class NormSpec:
 
 
 @dataclass(frozen=True)
+class LayerNormSpec:
+    """Layer norm over the last dimension: (x - mean) / sqrt(var + eps) * w + b, the variance the mean of the squared
+    deviations.  The bias is stored under the weight's name + `bias_suffix`."""
+    size: int
+    eps: float
+    bias_suffix: str = ".b"
+    kind: str = "layernorm"
+
+
+@dataclass(frozen=True)
 class PositionSpec:
     """How positions enter queries and keys.
 
@@ -42,7 +52,9 @@ class PositionSpec:
     divides every frequency by f (positions are read as position / f); ("yarn", factor, original, fast,
     slow) divides the frequencies of the pairs that make fewer than `slow` turns over `original` positions
     by `factor`, keeps those that make more than `fast`, ramps linearly between them, and multiplies cos
-    and sin by 0.1 ln(factor) + 1.  A law that has no entry in the position part is refused by name when
+    and sin by 0.1 ln(factor) + 1; ("llama3", factor, low, high, original) keeps the frequencies whose wavelength is
+    shorter than original / high, divides those whose wavelength is longer than original / low by `factor`, and blends
+    the two between them.  A law that has no entry in the position part is refused by name when
     the part is built.
     """
     kind: str = "rope"
@@ -74,6 +86,12 @@ class AttentionSpec:
     own_kv: bool = True                    # False: no key or value projection (nor the keys' norm): the layer's stop of the schedule reads
                                            # another stop's cache (`ScheduleEntry.cache_of`) with its own queries, window and scale
     reader_windows: Tuple[Optional[int], ...] = ()   # the windows of the stops that read this layer's cache: it keeps what the widest needs
+    mask_chunk: Optional[int] = None       # a query sees the keys of its own chunk of this many positions only (chunks counted from
+                                           # position 0 of the sequence), up to itself; the cache keeps every position
+    gate_per_head: bool = False            # with `gate`: one gate value a head ("g_proj.weight" is [n_heads, hidden])
+    qk_unit_norm: bool = False             # q and k are brought to unit root mean square a head, without a weight (`qk_norm` gives
+                                           # size and eps, no tensor is loaded).  A turn by position keeps a head's sum of
+                                           # squares, so the norm ahead of the turn and behind it are the same number
     kind: str = "attention"
 
     @property
@@ -88,7 +106,7 @@ class AttentionSpec:
     def kept_window(self) -> Optional[int]:
         """How many of the last positions the cache keeps: enough for this layer's window and for every reader's."""
         windows = (self.window,) + tuple(self.reader_windows)
-        return None if any(w is None for w in windows) else max(windows)
+        return None if self.mask_chunk or any(w is None for w in windows) else max(windows)
 
 
 @dataclass(frozen=True)
@@ -191,7 +209,10 @@ class LatentAttentionSpec:
     by the heads]; the latent is RMS-normed (`norm_eps`); a head's plain key is W_uk c, its value W_uv c
     (`v_dim` wide); score = (q_plain . k_plain + q_rot . k_rot) * scale.  Only the normed latent and the rotated
     key part are cached.  `position.rot_dim` of the `rot_dim` rotated features turn.  `gate`: the joined heads are
-    multiplied by sigmoid(W_g h) before the output projection."""
+    multiplied by sigmoid(W_g h) before the output projection (`gate_per_head`: one gate value a head, "g" is
+    [n_heads, hidden]).  `q_rank`: the queries come through a low-rank row of their own, q = W_uq rmsnorm(W_dq h) * w
+    (tensors "dq", "dq.norm", "uq" instead of "q").  `sink`: the softmax's denominator holds one more term exp(s_h), a
+    learned number a head (tensor "sink" [n_heads]) that has no key and no value and is not scaled."""
     hidden: int
     n_heads: int
     head_dim: int
@@ -204,6 +225,9 @@ class LatentAttentionSpec:
     gate: bool = True
     window: Optional[int] = None
     kind: str = "latent_attention"
+    q_rank: Optional[int] = None
+    sink: bool = False
+    gate_per_head: bool = False
 
 
 @dataclass(frozen=True)
@@ -228,7 +252,9 @@ class RoutedExpertsSpec:
     `identity`: the router has that many more outputs behind the experts'; one of them, chosen, stands for an expert
     that hands its input on.  `correction`: a tensor "correction" [experts + identity] is added to the scores for the
     choice only; the weights are the scores themselves.  `shared`: a `ClampedMlpSpec` that runs for every token beside
-    the chosen experts (tensors under "shared."), its output added."""
+    the chosen experts (tensors under "shared."), its output added; `shared_gate`: times sigmoid(W_sg h), one number a
+    token (tensor "shared.sg" [1, hidden], formed like a router's logit, in 32-bit).  `weight_on_input`: a chosen expert
+    runs on weight * h and its output is added as it is (instead of weight * expert(h))."""
     hidden: int
     intermediate: int
     experts: int
@@ -242,6 +268,8 @@ class RoutedExpertsSpec:
     correction: bool = False
     shared: Any = None
     kind: str = "routed_experts"
+    weight_on_input: bool = False
+    shared_gate: bool = False
 
 
 @dataclass(frozen=True)
@@ -263,6 +291,25 @@ class PostNormSpec:
     without the tensor leaves the step out."""
     alpha: float = 1.0
     bare_norm_name: Optional[str] = None
+
+
+@dataclass(frozen=True)
+class TokenSideSpec:
+    """What a token itself adds to the stream behind a layer: e = the layer's `dim` columns (from `offset`) of a second
+    embedding table's row for the token (`EmbeddingSpec.side_name`); y = W_proj (act(W_gate x) * e); x <- x +
+    rmsnorm(y) * w.  Tensors `prefix` + "gate" [dim, hidden], "proj" [hidden, dim], "norm" [hidden]."""
+    dim: int
+    offset: int
+    prefix: str
+    eps: float
+    activation: str = "gelu_tanh"
+
+
+@dataclass(frozen=True)
+class ParallelSpec:
+    """How a layer's sub-layers stand around a stream kept in 32-bit when both read ONE normed copy of it:
+    h = norm(x); x <- x + mixer(h) + ffn(h).  `side`: a `TokenSideSpec` whose row enters behind the sum."""
+    side: Any = None
 
 
 @dataclass(frozen=True)
@@ -289,7 +336,10 @@ class LayerSpec:
     order before the mixer, behind it, before the feed-forward, behind it; two norms for a layer without a feed-forward);
     "streams" is pre-norm around several residual streams (`residual`: a `StreamsSpec`) and takes a
     layer without a feed-forward (`ffn` None, one norm); "post_norm" norms the stream after every sum (`residual`: a
-    `PostNormSpec`; norms in the order behind the mixer, behind the feed-forward; one norm for a layer without one).  `norms[i]` loads its weight from `norm_names[i]`."""
+    `PostNormSpec`; norms in the order behind the mixer, behind the feed-forward; one norm for a layer without one);
+    "parallel" has ONE norm, whose output both sub-layers read, and adds their outputs together (`residual`: a
+    `ParallelSpec`).  `norms[i]` loads its weight from `norm_names[i]` (a norm with more tensors finds the others under
+    that name plus a suffix of its spec's)."""
     mixer: Any
     ffn: Any
     norms: Tuple[NormSpec, ...]
@@ -303,13 +353,16 @@ class LayerSpec:
 @dataclass(frozen=True)
 class EmbeddingSpec:
     """Token ids -> rows of the stream.  kind "embedding": a gather from a [vocab, hidden] table, times `scale`;
-    `wide`: the rows leave in 32-bit whatever the table is stored in (for a stream that is kept so)."""
+    `wide`: the rows leave in 32-bit whatever the table is stored in (for a stream that is kept so).  `side_name`: a
+    second table [vocab, side_width] whose rows for the step's tokens are handed to the layers (`TokenSideSpec`)."""
     vocab_size: int
     hidden: int
     name: str
     kind: str = "embedding"
     scale: float = 1.0
     wide: bool = False
+    side_name: Optional[str] = None
+    side_width: int = 0
 
 
 @dataclass(frozen=True)

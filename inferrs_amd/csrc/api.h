@@ -52,12 +52,15 @@ int ia_qk_rope_kv_strided(void* q_out, void* k_cache, void* v_cache, const void*
 
 // d: the keys' width, dv: the values' (v_cache [pages, nkv, dv, page_size], out [n, nq, dv])
 // sink: 1 adds exp(0) to the softmax's denominator (a key of score 0 that has no value); the same in the matrix-core kernels.
+// sinks: with sink, null or [nq] 32-bit values s_h, one a query head: the term is exp(s_h) instead (not scaled); mask_chunk > 0: a
+// query sees the keys of its own chunk of that many positions only (chunks counted from position 0), up to itself.
 // workspace: null, or ia_attention_generic_workspace(...) floats when that is not 0 (steps of few tokens: a wave a
 // segment of keys and a merge kernel, the same bits as without); max_kv_len: an upper bound of positions + 1
 int ia_attention_generic(void* out, const void* q, const void* k_cache, const void* v_cache,
                          const int* positions, const int* token_seq, const int* block_table,
                          int n, int max_pages, int nq, int nkv, int d, int dv, int page_size, int window,
-                         float scale, int dtype, float* workspace, int max_kv_len, int sink, hipStream_t stream);
+                         float scale, int dtype, float* workspace, int max_kv_len, int sink, int mask_chunk,
+                         const float* sinks, hipStream_t stream);
 long long ia_attention_generic_workspace(int n, int nq, int nkv, int d, int dv, int max_kv_len);
 
 int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, int in_dtype,
@@ -156,11 +159,11 @@ int ia_softcap(float* x, long long n, float cap, hipStream_t stream);
 int ia_latent_prep(void* q_out, void* k_cache, void* v_cache, const void* proj, const float* norm_w,
                    const float* cos_t, const float* sin_t, const int* slots, int n, int H, int d, int r,
                    int rank, int rd, int q_off, int down_off, int ld_proj, int page_size, float eps,
-                   float mag, int dtype, hipStream_t stream);
-// out[t][h][j] = sum_i w[h][j][i] x[t][h][i], optionally times sigmoid(gate[t][h][j])
+                   float mag, int interleaved, const void* qrows, int ld_q, int dtype, hipStream_t stream);
+// out[t][h][j] = sum_i w[h][j][i] x[t][h][i], optionally times sigmoid(gate[t][h][j]), or, with g_per_head, sigmoid(gate[t][h])
 int ia_head_product(void* out, const void* x, const void* w, const void* gate, int n, int H, int n_out,
                     int k_in, long long x_ld, int x_off, int x_head, long long o_ld, int o_off, int o_head,
-                    long long g_ld, int g_off, int x_dtype, int w_dtype, int out_dtype, hipStream_t stream);
+                    long long g_ld, int g_off, int g_per_head, int x_dtype, int w_dtype, int out_dtype, hipStream_t stream);
 
 // ---- gated linear recurrence behind a short convolution (recurrence.hip) ----------------------------------------
 // u_lo: null, or a bfloat16 copy of u (for products that take it in that precision)
@@ -189,13 +192,15 @@ int ia_rglru_scan_chunked(void* out, float* state, float* work, const float* u, 
 // choice_bias: null, or [E] 32-bit values that count in the choice only (score + bias picks, the score weighs).  The plan
 // gives a pair whose choice is E or beyond (an output of the router that names no expert with weights) no place and no tile.
 int ia_route(int* sel, float* weight, const void* h, const void* router, int n, int W, int E, int top,
-             float scale, int score_fn, int renorm, const float* choice_bias, int dtype, hipStream_t stream);
+             float scale, int score_fn, int renorm, const float* choice_bias, int gates, float* gate_out, int dtype,
+             hipStream_t stream);
 int ia_route_tiles(int pairs, int E);
 int ia_route_plan(int* order, int* tile_expert, int* tile_first, int* tile_rows, int* meta, const int* sel,
                   int pairs, int E, int tile, hipStream_t stream);
 int ia_experts_gate_up(void* act, const void* h, const void* w_gu, const int* order, const int* tile_expert,
                        const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int top,
-                       int W, int ff, float limit, float alpha, int tile, int tiled, int dtype, hipStream_t stream);
+                       int W, int ff, float limit, float alpha, int tile, int tiled, const float* in_weight, int dtype,
+                       hipStream_t stream);
 int ia_experts_down(float* y, const void* act, const void* w_down, const int* order, const int* tile_expert,
                     const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int W,
                     int ff, int tile, int tiled, int dtype, hipStream_t stream);
@@ -209,6 +214,17 @@ int ia_sandwich_step(float* x, const void* y1, float s1, const void* y2, float s
 // act over every element in place: 1 SiLU, 2 GELU in its tanh form, 3 the exact GELU
 int ia_activation(void* x, long long n, int act, int dtype, hipStream_t stream);
 
+// A 32-bit residual stream whose sub-layers all read one normed copy (parallel.hip): x += y1 + y2 + sum_k [routed_w[k]] routed[k]
+// + y3_scale y3; x += rmsnorm(enter) * enter_w; h = norm(x) (a layer norm with weight and bias, or with center 0 an RMS norm):
+// every part optional, one kernel.  y_dtype: of y1, y2, y3, enter; h_dtype: of xr (the new x once more) and h.  rows: only these
+// rows through the norm, nothing added, the stream left alone.
+int ia_parallel_step(float* x, const void* y1, const void* y2, const void* y3, int y1_splits, int y2_splits, int y3_splits,
+                     const float* y3_scale, const float* routed, const float* routed_w, int top, const void* enter,
+                     const float* enter_w, float enter_eps, void* xr, const float* norm_w, const float* norm_b, float norm_eps,
+                     int center, void* h, const int* rows, int n, int W, int y_dtype, int h_dtype, hipStream_t stream);
+// out[t][c] = act(g[t][c]) * e[t][e_off + c]; act: 1 SiLU, 2 GELU in its tanh form
+int ia_gate_rows(void* out, const void* g, const void* e, int rows, int cols, long long e_ld, int e_off, int act, int dtype,
+                 hipStream_t stream);
 // A 32-bit residual stream that is normed after every sum (postnorm.hip): x <- rmsnorm(alpha x + y + sum_k routed_w[k] *
 // routed[k] + y2) * w, written back in 32-bit and to h (h_dtype; null: not wanted); every addend may be null.  routed
 // [n, top, W] 32-bit with weights [n, top]; a pair whose sel (null: none) is real_experts or more stands for the stream's
@@ -221,7 +237,7 @@ int ia_postnorm_step(float* x, float alpha, const void* y, const void* y2, int y
 int ia_embed_gather_scaled(float* out, void* h, const void* table, const int* ids, int n, int hidden, int vocab,
                            float scale, int dtype, hipStream_t stream);
 // a[row][c] *= sigmoid(g[row * g_ld + g_off + c]) in place, a [rows, cols]
-int ia_sigmoid_gate(void* a, const void* g, int rows, int cols, int g_ld, int g_off, int dtype, hipStream_t stream);
+int ia_sigmoid_gate(void* a, const void* g, int rows, int cols, int g_ld, int g_off, int group, int dtype, hipStream_t stream);
 // rows of [gate | up] -> g' * sigmoid(slope g') * (u' + 1) with g' = min(gate, limit), u' = clamp(up, -limit, limit)
 int ia_clamped_gate_mul(void* out, const void* gu, int rows, int inter, float limit, float slope, int dtype,
                         hipStream_t stream);
@@ -268,7 +284,7 @@ int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_
                       const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
                       int n_tokens, int max_q_len, int max_kv_len, int max_pages,
                       int nq, int nkv, int d, int page_size, int window, float scale,
-                      int splits, int chunk, int sink, hipStream_t stream);
+                      int splits, int chunk, int sink, int mask_chunk, const float* sinks, hipStream_t stream);
 // Decode steps (one token a request, head sizes in steps of 64): per-head norm, rotation, cache write, attention
 // and the merge of the key splits in one kernel.  `workspace` holds ia_attention_decode_workspace() floats;
 // `counters` holds at least ia_attention_decode_counters() 32-bit words that are zero before the call and zero

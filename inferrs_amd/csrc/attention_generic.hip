@@ -66,7 +66,9 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
     int max_pages, int nq, int nkv, int d, int dv, int page_size, int window, float scale,
     float* __restrict__ partial,         // null: a wave walks all segments; else [n, nq, segs, dpad + 2], a wave a segment
     int segs,
-    int sink) {                          // 1: the softmax's denominator holds one more term, exp(0): a key of score 0 without a value
+    int sink,                            // 1: the softmax's denominator holds one more term, exp(0): a key of score 0 without a value
+    int mask_chunk,                      // > 0: a query sees the keys of its own chunk of this many positions only
+    const float* __restrict__ sinks) {   // with sink: null, or [nq] values s_h a query head; the term is exp(s_h), not scaled
     __shared__ __attribute__((aligned(16))) float stage[AG_TILE * AG_PITCH];     // keys: [key][dim]; values: [dim][key]
     __shared__ __attribute__((aligned(16))) float sp[HEADS][AG_TILE];
     extern __shared__ __attribute__((aligned(16))) float ag_rows[];       // queries, a segment's outputs, the totals: [HEADS][dpad] each
@@ -82,7 +84,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
     const int heads = kvh * g + g - h0 < HEADS ? kvh * g + g - h0 : HEADS;
     const int pos = positions[tok];
     const int* bt = block_table + (size_t)token_seq[tok] * max_pages;
-    const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+    const int lo = ia_key_floor(pos, window, mask_chunk);
     const int chunks = (d + AG_CHUNK - 1) / AG_CHUNK;                  // of a key's dimensions
     const int vchunks = (dv + AG_CHUNK - 1) / AG_CHUNK;                // of a value's
     const int dpad = (chunks > vchunks ? chunks : vchunks) * AG_CHUNK;
@@ -363,7 +365,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
     for (int h = 0; h < HEADS; ++h) {
         if (h >= heads) break;
         T* orow = out + ((size_t)tok * nq + h0 + h) * dv;
-        const float inv = 1.0f / (sink ? big_l[h] + expf(-big_m[h]) : big_l[h]);
+        const float inv = 1.0f / (sink ? big_l[h] + expf((sinks != nullptr ? sinks[h0 + h] : 0.f) - big_m[h]) : big_l[h]);
         for (int e = lane; e < dv; e += IA_WAVE) st(orow + e, st_[h * dpad + e] * inv);
     }
 }
@@ -372,11 +374,11 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
 template <typename T>
 __global__ __launch_bounds__(IA_WAVE) void attn_generic_merge_kernel(
     T* __restrict__ out, const float* __restrict__ partial, const int* __restrict__ positions, int nq, int d, int dpad,
-    int window, int segs, int sink) {
+    int window, int segs, int sink, int mask_chunk, const float* __restrict__ sinks) {
     const int lane = threadIdx.x;
     const int tok = blockIdx.x / nq, h = blockIdx.x - tok * nq;
     const int pos = positions[tok];
-    const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+    const int lo = ia_key_floor(pos, window, mask_chunk);
     float big_m = -INFINITY, big_l = 0.f;
     float big_o[AG_MAX_HEAD_DIM / IA_WAVE];
 #pragma unroll
@@ -395,7 +397,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_merge_kernel(
             if (e < dpad) big_o[t] = ag_merge_value(big_o[t], a, row[e], b);
         }
     }
-    const float inv = 1.0f / (sink ? big_l + expf(-big_m) : big_l);
+    const float inv = 1.0f / (sink ? big_l + expf((sinks != nullptr ? sinks[h] : 0.f) - big_m) : big_l);
     T* orow = out + ((size_t)tok * nq + h) * d;
 #pragma unroll
     for (int t = 0; t < AG_MAX_HEAD_DIM / IA_WAVE; ++t) {
@@ -421,7 +423,8 @@ extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cach
                                     const int* positions, const int* token_seq, const int* block_table,
                                     int n, int max_pages, int nq, int nkv, int d, int dv, int page_size,
                                     int window, float scale, int dtype, float* workspace, int max_kv_len,
-                                    int sink, hipStream_t stream) {
+                                    int sink, int mask_chunk, const float* sinks, hipStream_t stream) {
+    IA_CHECK(mask_chunk >= 0 && (sinks == nullptr || sink), "attention: mask_chunk %d must be >= 0 (0 = none), and sink values go with a sink", mask_chunk);
     IA_CHECK(n >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention: bad head counts nq=%d nkv=%d (n=%d)", nq, nkv, n);
     IA_CHECK(d > 0 && d <= AG_MAX_HEAD_DIM, "attention: head_dim %d is outside 1..%d", d, AG_MAX_HEAD_DIM);
     IA_CHECK(dv > 0 && dv <= AG_MAX_HEAD_DIM, "attention: the values' width %d is outside 1..%d", dv, AG_MAX_HEAD_DIM);
@@ -445,7 +448,7 @@ extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cach
     const bool vec = d % 4 == 0 && dv % 4 == 0 && page_size % 4 == 0 &&
                      (((uintptr_t)k_cache | (uintptr_t)v_cache) % (4 * elem)) == 0;
 #define AG_ARGS(T) (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache, positions, token_seq, block_table, max_pages, nq, nkv, \
-        d, dv, page_size, window, scale, workspace, segs, sink
+        d, dv, page_size, window, scale, workspace, segs, sink, mask_chunk, sinks
     // (a wave a segment, steps of few tokens: the operands are asked for a step ahead)
 #define AG_LAUNCH(T, V, H) do { \
         if (V && workspace != nullptr) attn_generic_kernel<T, V, H, true><<<grid, IA_WAVE, rows_bytes, stream>>>(AG_ARGS(T)); \
@@ -462,9 +465,9 @@ extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cach
     IA_LAUNCH_CHECK("attention_generic");
     if (workspace != nullptr) {
         if (dtype == IA_F32)
-            attn_generic_merge_kernel<float><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((float*)out, workspace, positions, nq, dv, dpad, window, segs, sink);
+            attn_generic_merge_kernel<float><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((float*)out, workspace, positions, nq, dv, dpad, window, segs, sink, mask_chunk, sinks);
         else
-            attn_generic_merge_kernel<bf16_t><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((bf16_t*)out, workspace, positions, nq, dv, dpad, window, segs, sink);
+            attn_generic_merge_kernel<bf16_t><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((bf16_t*)out, workspace, positions, nq, dv, dpad, window, segs, sink, mask_chunk, sinks);
         IA_LAUNCH_CHECK("attention_generic_merge");
     }
     return 0;

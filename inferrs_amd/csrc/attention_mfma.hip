@@ -83,9 +83,16 @@ struct AttnParams {
     float norm_eps;
     int norm_add_one;
     int sink;                   // 1: the softmax's denominator holds one more term, 2^(0 - m): a key of score 0 without a value
+    const float* sinks;         // with sink: null, or [nq] values s_h a query head (natural logarithm, not scaled): the term is 2^(s_h log2 e - m)
+    int mask_chunk;             // > 0: a query sees the keys of its own chunk of this many positions only, up to itself
 };
 
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
+
+// The sink's term of a row's denominator, in the kernels' log-2 domain: 2^(s_h log2 e - m), s_h = 0 without values.
+__device__ __forceinline__ float sink_term(const float* sinks, int head, float m) {
+    return exp2f((sinks != nullptr ? sinks[head] * 1.4426950408889634f : 0.f) - m);
+}
 
 // One column block (16 * NB columns) of one request and key/value head, over one split of the keys.
 template <int NB>
@@ -138,7 +145,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         for (int db = 0; db < DBV; ++db) acc[nb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
 
-    const int window_floor = p.window > 0 ? (pmin - p.window + 1 > 0 ? pmin - p.window + 1 : 0) : 0;   // first key any column sees
+    const int window_floor = ia_key_floor(pmin, p.window, p.mask_chunk);   // first key any column sees
     int lo = window_floor;
     int hi = pmax + 1;
     if (p.splits > 1) {
@@ -213,7 +220,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         for (int db = 0; db < DBV; ++db) op.v[db] = *(const uint4*)(vbase + (size_t)db * 16 * p.page);
     };
     auto compute_step = [&](Operands& op, int k0) {
-        const bool edge = k0 + 31 > pmin || (p.window > 0 && k0 < pmax - p.window + 1);
+        const bool edge = k0 + 31 > pmin || k0 < ia_key_floor(pmax, p.window, p.mask_chunk);
         if (k0 + 32 > kv_total) {
             // slots beyond the request's length hold anything at all: zero those values so that
             // a probability of zero times their content stays zero
@@ -229,7 +236,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
                 }
             }
         }
-        if (p.window > 0 && k0 < window_floor) {
+        if (k0 < window_floor) {
             // The walk starts at a multiple of 32 below the first key that any column sees: the keys in between
             // may lie in pages that the window has passed and the request has given back (the block table then
             // names some other page, which holds anything at all).  Their scores are masked below; their values
@@ -266,7 +273,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
                 for (int i = 0; i < 4; ++i) sc[4 * t + i] = s[t][i];
             if (edge) {
                 const int kbase_idx = k0 + 8 * G;
-                const int floor_key = p.window > 0 ? pos[nb] - p.window + 1 : 0;
+                const int floor_key = ia_key_floor(pos[nb], p.window, p.mask_chunk);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const int key = kbase_idx + j;
@@ -344,7 +351,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         if (!cvalid[nb]) continue;
         const size_t row = (size_t)(t0 + tq[nb]) * p.nq + head[nb];
         if (p.splits == 1) {
-            const float inv = 1.0f / (p.sink ? lt + exp2f(-m[nb]) : lt);
+            const float inv = 1.0f / (p.sink ? lt + sink_term(p.sinks, head[nb], m[nb]) : lt);
             bf16_t* o = p.out + row * HDV + 4 * G;
 #pragma unroll
             for (int db = 0; db < DBV; ++db) {
@@ -484,7 +491,7 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
         const bool cvalid = r < n_cols;
         const int head = kvh * g + col0 + (cvalid ? r : n_cols - 1);
 
-        const int window_floor = p.window > 0 ? (kv_start - p.window + 1 > 0 ? kv_start - p.window + 1 : 0) : 0;
+        const int window_floor = ia_key_floor(kv_start, p.window, p.mask_chunk);
         int lo = window_floor > c_lo ? window_floor : c_lo, hi = kv_total;
         if (p.splits > 1 && hi > c_lo + p.chunk) hi = c_lo + p.chunk;
         lo &= ~31;
@@ -645,7 +652,7 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
                     }
                 }
             }
-            if (p.window > 0 && k0 < window_floor) {
+            if (k0 < window_floor) {
                 // keys below the window may lie in pages that the request has given back: as above
                 const int first_good = window_floor - (k0 + 8 * G);
                 if (first_good > 0) {
@@ -697,7 +704,7 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) sc[4 * t + i] = s[t][i];
-            if (k0 + 31 > kv_start || (p.window > 0 && k0 < window_floor)) {
+            if (k0 + 31 > kv_start || (k0 < window_floor)) {
                 const int kbase_idx = k0 + 8 * G;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
@@ -794,7 +801,7 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
         const size_t row0 = (size_t)t0 * p.nq + kvh * g + col0;        // the block's first (token, head) row
         if (p.splits == 1) {
             if (!cvalid) return;
-            const float inv = 1.0f / (p.sink ? lt + exp2f(-m) : lt);
+            const float inv = 1.0f / (p.sink ? lt + sink_term(p.sinks, head, m) : lt);
             bf16_t* o = p.out + (row0 + r) * HD + 4 * G;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
@@ -835,7 +842,7 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
                 total = fmaf(team_ml[(w * n_cols + col) * 2 + 1], wt, total);
             }
             if (teams == 1) {
-                const float inv = 1.0f / (p.sink ? total + exp2f(-mx) : total);
+                const float inv = 1.0f / (p.sink ? total + sink_term(p.sinks, (int)((row0 + col) % p.nq), mx) : total);
                 uint2 w;
                 w.x = pack_bf16x2(o[0] * inv, o[1] * inv);
                 w.y = pack_bf16x2(o[2] * inv, o[3] * inv);
@@ -919,7 +926,7 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
             } else if (!active) {
                 continue;
             }
-            const float inv = 1.0f / (p.sink ? total + exp2f(-mx) : total);
+            const float inv = 1.0f / (p.sink ? total + sink_term(p.sinks, (int)((row0 + col) % p.nq), mx) : total);
             uint2 w;
             w.x = pack_bf16x2(o[0] * inv, o[1] * inv);
             w.y = pack_bf16x2(o[2] * inv, o[3] * inv);
@@ -1019,7 +1026,7 @@ void attn_tile_kernel(const AttnParams p) {
         const int* bt = p.block_table + (size_t)seq * p.max_pages;
         const int blast = (bcol0 + TILE_COLS <= n_cols ? bcol0 + TILE_COLS : n_cols) - 1;
         const int bpmin = kv_start + bcol0 / g, bpmax = kv_start + blast / g;
-        const int bfloor = p.window > 0 ? (bpmin - p.window + 1 > 0 ? bpmin - p.window + 1 : 0) : 0;   // first key the block sees
+        const int bfloor = ia_key_floor(bpmin, p.window, p.mask_chunk);   // first key the block sees
         int lo = bfloor;
         lo &= ~(TILE_STAGE - 1);
         int hi = bpmax + 1;
@@ -1046,7 +1053,7 @@ void attn_tile_kernel(const AttnParams p) {
         }
         const int wlast = (col0 + WAVE_COLS <= n_cols ? col0 + WAVE_COLS : n_cols) - 1;
         const int pmin = kv_start + (has_cols ? col0 : 0) / g, pmax = has_cols ? kv_start + wlast / g : -1;
-        const int wlo = p.window > 0 ? (pmin - p.window + 1 > 0 ? pmin - p.window + 1 : 0) : 0;
+        const int wlo = ia_key_floor(pmin, p.window, p.mask_chunk);
 
         uint4 qreg[NBW][KS];
 #pragma unroll
@@ -1198,7 +1205,7 @@ void attn_tile_kernel(const AttnParams p) {
                     for (int i = 0; i < 4; ++i) sc[4 * t + i] = sacc[t][i];
                 if constexpr (EDGE) {
                     const int kbase_idx = k0 + 8 * G;
-                    const int floor_key = p.window > 0 ? pos[nb] - p.window + 1 : 0;
+                    const int floor_key = ia_key_floor(pos[nb], p.window, p.mask_chunk);
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
                         const int key = kbase_idx + j;
@@ -1307,7 +1314,7 @@ void attn_tile_kernel(const AttnParams p) {
                 if (u == 1 && more && kg != 0) issue(other, page_l, off_l);
                 if (!live[u]) continue;
                 const int k0 = kb + 32 * u;
-                const bool edge = k0 + 31 > pmin || (p.window > 0 && k0 < pmax - p.window + 1);
+                const bool edge = k0 + 31 > pmin || k0 < ia_key_floor(pmax, p.window, p.mask_chunk);
                 if (edge) step(std::true_type(), u);
                 else step(std::false_type(), u);
             }
@@ -1371,7 +1378,7 @@ void attn_tile_kernel(const AttnParams p) {
             if (!cvalid[nb]) continue;
             const size_t row = (size_t)(t0 + tq[nb]) * p.nq + head[nb];
             if (p.splits == 1) {
-                const float inv = 1.0f / (p.sink ? lt + exp2f(-m[nb]) : lt);
+                const float inv = 1.0f / (p.sink ? lt + sink_term(p.sinks, head[nb], m[nb]) : lt);
                 bf16_t* o = p.out + row * HDV + 4 * G;
 #pragma unroll
                 for (int db = 0; db < DBV; ++db) {
@@ -1420,7 +1427,7 @@ static int attn_cus() {
 #define MERGE_WAVES 16
 __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
     bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
-    size_t first_row, int sink) {
+    size_t first_row, int sink, const float* __restrict__ sinks, int nq) {
     constexpr int PER = (HDV + IA_WAVE - 1) / IA_WAVE;
     __shared__ float weight[256];
     __shared__ float red[MERGE_WAVES][PER * IA_WAVE];
@@ -1452,7 +1459,7 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
             total += ml[2 * s + 1] * w;
         }
         total = wave_sum(total);
-        if (lane == 0) s_total = sink ? total + exp2f(-mx) : total;
+        if (lane == 0) s_total = sink ? total + sink_term(sinks, (int)(row % nq), mx) : total;
     }
     __syncthreads();
     float o[PER];
@@ -1490,7 +1497,7 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
 #define MERGE_ROWS_FROM 1024
 __global__ __launch_bounds__(MERGE_ROWS_WAVES * IA_WAVE) void attn_merge_rows_kernel(
     bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
-    size_t first_row, size_t n_rows, int sink) {
+    size_t first_row, size_t n_rows, int sink, const float* __restrict__ sinks, int nq) {
     constexpr int PER = (HDV + IA_WAVE - 1) / IA_WAVE;
     const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
     const size_t local = (size_t)blockIdx.x * MERGE_ROWS_WAVES + wave;
@@ -1513,7 +1520,7 @@ __global__ __launch_bounds__(MERGE_ROWS_WAVES * IA_WAVE) void attn_merge_rows_ke
             if (e < HDV) o[t] = fmaf(po[(size_t)s * HDV + e], w, o[t]);
         }
     }
-    const float inv = 1.0f / (sink ? total + exp2f(-mx) : total);
+    const float inv = 1.0f / (sink ? total + sink_term(sinks, (int)(row % nq), mx) : total);
 #pragma unroll
     for (int t = 0; t < PER; ++t) {
         const int e = lane + t * IA_WAVE;
@@ -1568,7 +1575,8 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
                             const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
                             int n_tokens, int max_q_len, int max_kv_len, int max_pages,
                             int nq, int nkv, int d, int page_size, int window, float scale,
-                            int splits, int chunk, int sink, const FusedArgs* fused, hipStream_t stream) {
+                            int splits, int chunk, int sink, int mask_chunk, const float* sinks, const FusedArgs* fused,
+                            hipStream_t stream) {
     IA_CHECK(d == HD, "attention_mfma: built for head_dim %d, called with %d", HD, d);
     IA_CHECK(n >= 0 && n_seqs >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0,
              "attention_mfma: bad sizes n=%d seqs=%d nq=%d nkv=%d", n, n_seqs, nq, nkv);
@@ -1602,6 +1610,8 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
     p.splits = splits; p.chunk = chunk; p.seq_begin = seq_begin; p.token_begin = token_begin;
     p.scale_log2 = scale * 1.4426950408889634f;
     p.sink = sink ? 1 : 0;
+    IA_CHECK(mask_chunk >= 0 && (sinks == nullptr || sink), "attention_mfma: mask_chunk %d must be >= 0 (0 = none), and sink values go with a sink", mask_chunk);
+    p.sinks = sinks; p.mask_chunk = mask_chunk;
     const long long cols = (long long)max_q_len * g;
     // Columns a wave: 16 for decode, 32 for portions of prompts.  (64 keep every loaded key and
     // value in use for twice as many products but need the registers of a whole SIMD; with 32
@@ -1664,10 +1674,10 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         if (rows >= MERGE_ROWS_FROM && splits <= 16)
             attn_merge_rows_kernel<<<(unsigned)((rows + MERGE_ROWS_WAVES - 1) / MERGE_ROWS_WAVES), MERGE_ROWS_WAVES * IA_WAVE,
                                      0, stream>>>((bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq,
-                                                  (size_t)rows, p.sink);
+                                                  (size_t)rows, p.sink, p.sinks, nq);
         else
             attn_merge_kernel<<<(unsigned)rows, MERGE_WAVES * IA_WAVE, 0, stream>>>(
-                (bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq, p.sink);
+                (bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq, p.sink, p.sinks, nq);
         IA_LAUNCH_CHECK("attention_merge");
     }
     return 0;
@@ -1678,10 +1688,11 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
                                  const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
                                  int n_tokens, int max_q_len, int max_kv_len, int max_pages,
                                  int nq, int nkv, int d, int page_size, int window, float scale,
-                                 int splits, int chunk, int sink, hipStream_t stream) {
+                                 int splits, int chunk, int sink, int mask_chunk, const float* sinks,
+                                 hipStream_t stream) {
     return attention_launch(out, workspace, q, k_cache, v_cache, block_table, cu_tokens, positions, n, seq_begin,
                             n_seqs, token_begin, n_tokens, max_q_len, max_kv_len, max_pages, nq, nkv, d, page_size,
-                            window, scale, splits, chunk, sink, nullptr, stream);
+                            window, scale, splits, chunk, sink, mask_chunk, sinks, nullptr, stream);
 }
 
 // Whether this head size has the fused decode form.
@@ -1708,5 +1719,5 @@ extern "C" int ia_attention_mfma_decode_fused(void* out, float* workspace, const
     const FusedArgs fused = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, slots, eps, add_one, counters, n_counters};
     return attention_launch(out, workspace, nullptr, k_cache, v_cache, block_table, cu_tokens, positions, n, seq_begin,
                             n_seqs, token_begin, n_tokens, 1, max_kv_len, max_pages, nq, nkv, d, page_size,
-                            window, scale, splits, chunk, sink, &fused, stream);
+                            window, scale, splits, chunk, sink, 0, nullptr, &fused, stream);
 }

@@ -55,6 +55,20 @@ __device__ __forceinline__ float gate_act(float g, int act) {
     return g / (1.0f + expf(-g));
 }
 
+// ---- which keys a query sees ---------------------------------------------------------------------
+// The first key that the query at `pos` sees (it sees every key from there up to itself).  window > 0: the last `window`
+// positions, itself included; mask_chunk > 0: the keys of its own chunk of `mask_chunk` positions, chunks counted from
+// position 0 of the sequence; both 0: every key.  The floor never falls as `pos` grows, which is what the kernels that
+// walk the keys of several queries together rest on.
+__host__ __device__ __forceinline__ int ia_key_floor(int pos, int window, int mask_chunk) {
+    int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    if (mask_chunk > 0) {
+        const int c = pos - pos % mask_chunk;
+        lo = c > lo ? c : lo;
+    }
+    return lo;
+}
+
 // ---- reductions -----------------------------------------------------------------------------
 // Butterfly over the 64 lanes: every lane ends with the same value, and the order of the
 // additions is fixed by the lane numbers alone.

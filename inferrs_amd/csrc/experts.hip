@@ -48,7 +48,10 @@ template <typename T, bool VEC, int SHARE = IA_ROUTE_SHARE, int WAVES = IA_ROUTE
 __global__ __launch_bounds__(64 * WAVES) void route_kernel(int* __restrict__ sel, float* __restrict__ weight,
                                                                     const T* __restrict__ h, const T* __restrict__ wr, int n,
                                                                     int W, int E, int top, float scale, int score_fn,
-                                                                    int renorm, const float* __restrict__ choice_bias) {
+                                                                    int renorm, const float* __restrict__ choice_bias,
+                                                                    int gates, float* __restrict__ gate_out) {
+    // E counts every row of the router's matrix: the last `gates` of them take no part in the choice; the sigmoid of
+    // such a row's logit is handed out as it is (gate_out [n, gates]): a gate a token, formed like a router's logit.
     __shared__ float logits[IA_MAX_EXPERTS];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const T* row = h + (long long)t * W;
@@ -89,6 +92,10 @@ __global__ __launch_bounds__(64 * WAVES) void route_kernel(int* __restrict__ sel
     }
     __syncthreads();
     if (wave != 0) return;
+    if (gates > 0) {
+        E -= gates;
+        for (int j = lane; j < gates; j += IA_WAVE) gate_out[(long long)t * gates + j] = 1.0f / (1.0f + expf(-logits[E + j]));
+    }
     float z[IA_MAX_EXPERTS / IA_WAVE];             // expert e lives in lane e % 64, register e / 64
 #pragma unroll
     for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) {
@@ -200,7 +207,7 @@ __global__ __launch_bounds__(1024) void route_plan_kernel(int* __restrict__ orde
 }
 
 // act[place][j] = g' * sigmoid(alpha g') * (u' + 1), g' = min(gate_j . x, limit), u' = clamp(up_j . x, -limit, limit);
-// x = h[pair / top].  w_gu [E][2 ff][W]: an expert's gate rows, then its up rows.
+// x = h[pair / top] (times in_weight[pair], where given: 32-bit, one a pair).  w_gu [E][2 ff][W]: an expert's gate rows, then its up rows.
 template <typename T>
 __global__ __launch_bounds__(256) void experts_gate_up_kernel(T* __restrict__ act, const T* __restrict__ h,
                                                               const T* __restrict__ w_gu, const int* __restrict__ order,
@@ -208,7 +215,7 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(T* __restrict__ ac
                                                               const int* __restrict__ tile_first,
                                                               const int* __restrict__ tile_rows,
                                                               const int* __restrict__ meta, int top, int W, int ff,
-                                                              float limit, float alpha) {
+                                                              float limit, float alpha, const float* __restrict__ in_weight) {
     __shared__ TileShared sh;
     const int tile = blockIdx.y;
     if (tile >= meta[0]) return;
@@ -226,7 +233,9 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(T* __restrict__ ac
         for (int b = 0; b < 4; ++b) {
             const int j = col0 + 4 * tx + b;
             if (j >= ff) continue;
-            const float gv = fminf(g[a][b], limit), uv = fminf(fmaxf(u[a][b], -limit), limit);
+            // (in_weight: the pair's weight is a factor on the expert's INPUT, hence on both sums ahead of the limits)
+            const float wi = in_weight != nullptr ? in_weight[order[first + i]] : 1.0f;
+            const float gv = fminf(g[a][b] * wi, limit), uv = fminf(fmaxf(u[a][b] * wi, -limit), limit);
             st(act + (long long)(first + i) * ff + j, gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
         }
     }
@@ -272,7 +281,7 @@ __global__ __launch_bounds__(256) void experts_gate_up_mfma_kernel(bf16_t* __res
                                                                    const int* __restrict__ tile_first,
                                                                    const int* __restrict__ tile_rows,
                                                                    const int* __restrict__ meta, int top, int W, int ff,
-                                                                   float limit, float alpha) {
+                                                                   float limit, float alpha, const float* __restrict__ in_weight) {
     using Tile = TileMfma<RT, FT, 64, true>;
     __shared__ typename Tile::Shared sh;
     const int tile = blockIdx.y;
@@ -296,7 +305,8 @@ __global__ __launch_bounds__(256) void experts_gate_up_mfma_kernel(bf16_t* __res
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 if (i >= rows || j0 + q >= ff) continue;
-                const float gv = fminf(gs[q], limit), uv = fminf(fmaxf(us[q], -limit), limit);
+                const float wi = in_weight != nullptr ? in_weight[order[first + i]] : 1.0f;
+                const float gv = fminf(gs[q] * wi, limit), uv = fminf(fmaxf(us[q] * wi, -limit), limit);
                 st(act + (long long)(first + i) * ff + j0 + q, gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
             }
         }
@@ -329,13 +339,17 @@ __global__ __launch_bounds__(256) void experts_down_mfma_kernel(float* __restric
 
 // choice_bias: null, or [E] 32-bit values added to the scores for the choice only (the weights are the scores themselves)
 extern "C" int ia_route(int* sel, float* weight, const void* h, const void* router, int n, int W, int E, int top,
-                        float scale, int score_fn, int renorm, const float* choice_bias, int dtype, hipStream_t stream) {
-    IA_CHECK(n >= 0 && W > 0 && E >= 1 && E <= IA_MAX_EXPERTS && top >= 1 && top <= E && top <= IA_MAX_TOP,
-             "route: n=%d width=%d experts=%d (up to %d) top=%d (up to %d)", n, W, E, IA_MAX_EXPERTS, top, IA_MAX_TOP);
+                        float scale, int score_fn, int renorm, const float* choice_bias, int gates, float* gate_out,
+                        int dtype, hipStream_t stream) {
+    // E: the router's outputs that can be chosen; the matrix holds `gates` more rows behind them (see the kernel)
+    IA_CHECK(gates >= 0 && (gates == 0 || gate_out != nullptr), "route: %d gate rows need a place for their values", gates);
+    IA_CHECK(n >= 0 && W > 0 && E >= 1 && E + gates <= IA_MAX_EXPERTS && top >= 1 && top <= E && top <= IA_MAX_TOP,
+             "route: n=%d width=%d experts=%d and %d gate rows (up to %d) top=%d (up to %d)", n, W, E, gates, IA_MAX_EXPERTS, top, IA_MAX_TOP);
+    E += gates;
     IA_CHECK(score_fn == IA_SCORE_SIGMOID || score_fn == IA_SCORE_SOFTMAX, "route: unknown score function %d", score_fn);
     if (n == 0) return 0;
     const bool vec = W % 8 == 0 && tile_mfma_aligned(h) && tile_mfma_aligned(router);
-#define IA_ROUTE_SW(T, V, S, WV) route_kernel<T, V, S, WV><<<n, 64 * WV, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm, choice_bias)
+#define IA_ROUTE_SW(T, V, S, WV) route_kernel<T, V, S, WV><<<n, 64 * WV, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm, choice_bias, gates, gate_out)
 #define IA_ROUTE_S(T, V, S) IA_ROUTE_SW(T, V, S, IA_ROUTE_WAVES)
     // (up to 32 outputs: 8 a wave; up to 64: as many a wave as take them all in one walk over the row.  A step of few
     // tokens has few blocks, and a wave's walk is a chain of trips to the memory: sixteen waves a token then, each with
@@ -370,7 +384,8 @@ extern "C" int ia_route_plan(int* order, int* tile_expert, int* tile_first, int*
 
 extern "C" int ia_experts_gate_up(void* act, const void* h, const void* w_gu, const int* order, const int* tile_expert,
                                   const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int top,
-                                  int W, int ff, float limit, float alpha, int tile, int tiled, int dtype, hipStream_t stream) {
+                                  int W, int ff, float limit, float alpha, int tile, int tiled, const float* in_weight, int dtype,
+                                  hipStream_t stream) {
     IA_CHECK(pairs >= 0 && W > 0 && ff > 0 && top >= 1 && limit > 0.f && (tile == 32 || tile == 64 || tile == 128), "experts_gate_up: bad sizes");
     if (pairs == 0) return 0;
     IA_CHECK(!tiled || (dtype == IA_BF16 && W % 8 == 0 && tile_mfma_aligned(h) && tile_mfma_aligned(w_gu)),
@@ -381,19 +396,19 @@ extern "C" int ia_experts_gate_up(void* act, const void* h, const void* w_gu, co
     IA_CHECK(grid.y <= 65535, "experts_gate_up: %u row tiles are more than a grid takes", grid.y);
     if (tiled && tile == 128)
         experts_gate_up_mfma_kernel<8, 2><<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, order,
-                                                                    tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+                                                                    tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha, in_weight);
     else if (tiled && tile == 64)
         experts_gate_up_mfma_kernel<4, 2><<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, order,
-                                                                    tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+                                                                    tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha, in_weight);
     else if (tiled)
         experts_gate_up_mfma_kernel<2, 1><<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, order,
-                                                                    tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+                                                                    tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha, in_weight);
     else if (dtype == IA_F32)
         experts_gate_up_kernel<float><<<grid, 256, 0, stream>>>((float*)act, (const float*)h, (const float*)w_gu, order,
-                                                                tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+                                                                tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha, in_weight);
     else
         experts_gate_up_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, order,
-                                                                 tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+                                                                 tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha, in_weight);
     IA_LAUNCH_CHECK("experts_gate_up");
     return 0;
 }

@@ -15,14 +15,15 @@
 
 // proj[t] = [.. q (H x (d + r)) at q_off .. | down (rank + r) at down_off ..]; q_out [n, H, rank + r] gets the
 // rotated parts at [rank, rank + r).  Of a rotated part the first `rd` features turn (i paired with i + rd / 2), the
-// rest pass.  cos / sin [n, rd / 2] are multiplied by `mag`.  The key row goes to k_cache [pages][page][D] and, once
+// rest pass (`interleaved`: 2 i paired with 2 i + 1 instead).  cos / sin [n, rd / 2] are multiplied by `mag`.  The key row goes to k_cache [pages][page][D] and, once
 // more, transposed to v_cache [pages][D][page] (D = rank + r), at slot slots[t]; slots null: no cache write.
 template <typename T>
 __global__ __launch_bounds__(256) void latent_prep_kernel(
     T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, const T* __restrict__ proj,
     const float* __restrict__ norm_w, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ slots, int H, int d, int r, int rank, int rd, int q_off, int down_off, int ld_proj,
-    int page_size, float eps, float mag) {
+    int page_size, float eps, float mag, int interleaved, const T* __restrict__ qrows, int ld_q) {
+    // qrows: null, or the queries' rows where they are no part of `proj` (a product of their own): [n, ld_q], q at q_off
     __shared__ float scratch[16];
     const int t = blockIdx.x;
     const int D = rank + r, half = rd / 2;
@@ -49,9 +50,12 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
                 const int i = j - rank;
                 const T* kr = down + rank;
                 if (cs != nullptr && i < rd) {
-                    const int p = i < half ? i : i - half;
-                    const float a = ld(kr + p), b = ld(kr + p + half), c = cs[p] * mag, s = sn[p] * mag;
-                    v = i < half ? a * c - b * s : b * c + a * s;
+                    // (pair p: features p and p + rd / 2, or, interleaved, 2 p and 2 p + 1; `first`: this is the pair's first)
+                    const bool first = interleaved ? (i & 1) == 0 : i < half;
+                    const int p = interleaved ? i >> 1 : (i < half ? i : i - half);
+                    const int ia = interleaved ? 2 * p : p, ib = interleaved ? 2 * p + 1 : p + half;
+                    const float a = ld(kr + ia), b = ld(kr + ib), c = cs[p] * mag, s = sn[p] * mag;
+                    v = first ? a * c - b * s : b * c + a * s;
                 } else {
                     v = ld(kr + i);
                 }
@@ -62,12 +66,14 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
     }
     for (int idx = threadIdx.x; idx < H * r; idx += blockDim.x) {
         const int hh = idx / r, i = idx - hh * r;
-        const T* qr = row + q_off + (long long)hh * (d + r) + d;
+        const T* qr = (qrows != nullptr ? qrows + (long long)t * ld_q : row) + q_off + (long long)hh * (d + r) + d;
         float v;
         if (cs != nullptr && i < rd) {
-            const int p = i < half ? i : i - half;
-            const float a = ld(qr + p), b = ld(qr + p + half), c = cs[p] * mag, s = sn[p] * mag;
-            v = i < half ? a * c - b * s : b * c + a * s;
+            const bool first = interleaved ? (i & 1) == 0 : i < half;
+            const int p = interleaved ? i >> 1 : (i < half ? i : i - half);
+            const int ia = interleaved ? 2 * p : p, ib = interleaved ? 2 * p + 1 : p + half;
+            const float a = ld(qr + ia), b = ld(qr + ib), c = cs[p] * mag, s = sn[p] * mag;
+            v = first ? a * c - b * s : b * c + a * s;
         } else {
             v = ld(qr + i);
         }
@@ -78,11 +84,11 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
 extern "C" int ia_latent_prep(void* q_out, void* k_cache, void* v_cache, const void* proj, const float* norm_w,
                               const float* cos_t, const float* sin_t, const int* slots, int n, int H, int d, int r,
                               int rank, int rd, int q_off, int down_off, int ld_proj, int page_size, float eps,
-                              float mag, int dtype, hipStream_t stream) {
+                              float mag, int interleaved, const void* qrows, int ld_q, int dtype, hipStream_t stream) {
     IA_CHECK(n >= 0 && H > 0 && d > 0 && r >= 0 && rank > 0 && rd >= 0 && rd <= r && rd % 2 == 0 && page_size > 0,
              "latent_prep: bad sizes n=%d heads=%d dim=%d rot_dim=%d rank=%d rotated=%d page=%d", n, H, d, r, rank, rd,
              page_size);
-    IA_CHECK(q_off >= 0 && down_off >= 0 && q_off + H * (d + r) <= ld_proj && down_off + rank + r <= ld_proj,
+    IA_CHECK(q_off >= 0 && down_off >= 0 && q_off + H * (d + r) <= (qrows != nullptr ? ld_q : ld_proj) && down_off + rank + r <= ld_proj,
              "latent_prep: the projections' row of %d does not hold q at %d and the latent row at %d", ld_proj, q_off,
              down_off);
     IA_CHECK(slots == nullptr || (k_cache != nullptr && v_cache != nullptr), "latent_prep: slots without a cache");
@@ -92,11 +98,11 @@ extern "C" int ia_latent_prep(void* q_out, void* k_cache, void* v_cache, const v
     if (dtype == IA_F32)
         latent_prep_kernel<float><<<n, 256, 0, stream>>>((float*)q_out, (float*)k_cache, (float*)v_cache,
                                                          (const float*)proj, norm_w, cos_t, sin_t, slots, H, d, r, rank, rd,
-                                                         q_off, down_off, ld_proj, page_size, eps, mag);
+                                                         q_off, down_off, ld_proj, page_size, eps, mag, interleaved, (const float*)qrows, ld_q);
     else
         latent_prep_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                                                           (const bf16_t*)proj, norm_w, cos_t, sin_t, slots, H, d, r, rank,
-                                                          rd, q_off, down_off, ld_proj, page_size, eps, mag);
+                                                          rd, q_off, down_off, ld_proj, page_size, eps, mag, interleaved, (const bf16_t*)qrows, ld_q) ;
     IA_LAUNCH_CHECK("latent_prep");
     return 0;
 }
@@ -109,7 +115,7 @@ template <typename TX, typename TW, typename TO>
 __global__ __launch_bounds__(256) void head_product_kernel(
     TO* __restrict__ out, const TX* __restrict__ x, const TW* __restrict__ w, const TX* __restrict__ gate, int n,
     int n_out, int k_in, long long x_ld, int x_off, int x_head, long long o_ld, int o_off, int o_head, long long g_ld,
-    int g_off) {
+    int g_off, int g_per_head) {
     __shared__ TileShared sh;
     const int h = blockIdx.z, row0 = blockIdx.y * IA_TM, col0 = blockIdx.x * IA_TN;
     float acc[2][4], acc2[2][4];
@@ -128,7 +134,7 @@ __global__ __launch_bounds__(256) void head_product_kernel(
             if (j >= n_out) continue;
             float v = acc[a][b];
             if (gate != nullptr) {
-                const float g = ld(gate + (long long)t * g_ld + g_off + (long long)h * n_out + j);
+                const float g = ld(gate + (long long)t * g_ld + g_off + (g_per_head ? h : (long long)h * n_out + j));
                 v = v / (1.0f + expf(-g));
             }
             st(out + (long long)t * o_ld + o_off + (long long)h * o_head + j, v);
@@ -141,7 +147,7 @@ template <typename TO, int RT, int FT, int KC>
 __global__ __launch_bounds__(256) void head_product_mfma_kernel(
     TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const bf16_t* __restrict__ gate, int n,
     int n_out, int k_in, long long x_ld, int x_off, int x_head, long long o_ld, int o_off, int o_head, long long g_ld,
-    int g_off) {
+    int g_off, int g_per_head) {
     using Tile = TileMfma<RT, FT, KC, false>;
     __shared__ typename Tile::Shared sh;
     const int h = blockIdx.z, row0 = blockIdx.y * Tile::ROWS, col0 = blockIdx.x * Tile::FEATURES;
@@ -155,7 +161,7 @@ __global__ __launch_bounds__(256) void head_product_mfma_kernel(
         if (t >= n || j >= n_out) return;
         float v = acc[ft][rt][q];
         if (gate != nullptr) {
-            const float g = ld(gate + (long long)t * g_ld + g_off + (long long)h * n_out + j);
+            const float g = ld(gate + (long long)t * g_ld + g_off + (g_per_head ? h : (long long)h * n_out + j));
             v = v / (1.0f + expf(-g));
         }
         st(out + (long long)t * o_ld + o_off + (long long)h * o_head + j, v);
@@ -167,20 +173,21 @@ __global__ __launch_bounds__(256) void head_product_mfma_kernel(
 // 8 run on the matrix cores, the rest on the vector units.
 extern "C" int ia_head_product(void* out, const void* x, const void* w, const void* gate, int n, int H, int n_out,
                                int k_in, long long x_ld, int x_off, int x_head, long long o_ld, int o_off, int o_head,
-                               long long g_ld, int g_off, int x_dtype, int w_dtype, int out_dtype, hipStream_t stream) {
+                               long long g_ld, int g_off, int g_per_head, int x_dtype, int w_dtype, int out_dtype,
+                               hipStream_t stream) {
     IA_CHECK(n >= 0 && H > 0 && n_out > 0 && k_in > 0, "head_product: bad sizes n=%d heads=%d out=%d in=%d", n, H, n_out,
              k_in);
     IA_CHECK(x_off >= 0 && o_off >= 0 && x_off + (long long)(H - 1) * x_head + k_in <= x_ld &&
                  o_off + (long long)(H - 1) * o_head + n_out <= o_ld,
              "head_product: the heads do not fit rows of %lld and %lld", x_ld, o_ld);
-    IA_CHECK(gate == nullptr || (g_off >= 0 && g_off + (long long)H * n_out <= g_ld), "head_product: the gate does not fit its row");
+    IA_CHECK(gate == nullptr || (g_off >= 0 && g_off + (long long)H * (g_per_head ? 1 : n_out) <= g_ld), "head_product: the gate does not fit its row");
     IA_CHECK(H <= 65535, "head_product: %d heads are more than a grid takes", H);
     if (n == 0) return 0;
     const dim3 grid((n_out + IA_TN - 1) / IA_TN, (n + IA_TM - 1) / IA_TM, H);
 #define IA_LAUNCH(TX, TW, TO)                                                                                        \
     head_product_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((TO*)out, (const TX*)x, (const TW*)w, (const TX*)gate, n, \
                                                               n_out, k_in, x_ld, x_off, x_head, o_ld, o_off, o_head,  \
-                                                              g_ld, g_off)
+                                                              g_ld, g_off, g_per_head)
     const bool cores = x_dtype == IA_BF16 && w_dtype == IA_BF16 && k_in % 8 == 0 && x_ld % 8 == 0 && x_off % 8 == 0 &&
                        x_head % 8 == 0 && tile_mfma_aligned(x) && tile_mfma_aligned(w);
     // many rows and wide heads: tiles of 64 rows x 128 features (every operand read serves more products)
@@ -189,7 +196,7 @@ extern "C" int ia_head_product(void* out, const void* x, const void* w, const vo
 #define IA_CORES(TO, RT, FT, KC, G)                                                                                            \
     head_product_mfma_kernel<TO, RT, FT, KC><<<G, 256, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w,                 \
                                                                     (const bf16_t*)gate, n, n_out, k_in, x_ld, x_off, x_head,    \
-                                                                    o_ld, o_off, o_head, g_ld, g_off)
+                                                                    o_ld, o_off, o_head, g_ld, g_off, g_per_head)
     if (cores && out_dtype == IA_BF16 && large) IA_CORES(bf16_t, 4, 2, 64, big);
     else if (cores && out_dtype == IA_BF16) IA_CORES(bf16_t, 2, 1, 64, grid);
     else if (cores && out_dtype == IA_F32 && large) IA_CORES(float, 4, 2, 64, big);

@@ -250,11 +250,12 @@ extern "C" int ia_embed_gather_scaled(float* out, void* h, const void* table, co
 
 // ---- a[row][c] *= sigmoid(g[row][g_off + c]) in place ------------------------------------------------------------------
 template <typename T>
-__global__ void sigmoid_gate_kernel(T* __restrict__ a, const T* __restrict__ g, int cols, int g_ld, int g_off, size_t total) {
+__global__ void sigmoid_gate_kernel(T* __restrict__ a, const T* __restrict__ g, int cols, int g_ld, int g_off, int group,
+                                    size_t total) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t row = i / cols;
         const int c = (int)(i - row * cols);
-        const float z = ld(g + row * g_ld + g_off + c);
+        const float z = ld(g + row * g_ld + g_off + c / group);
         st(a + i, ld(a + i) / (1.0f + expf(-z)));
     }
 }
@@ -280,13 +281,15 @@ __global__ void sigmoid_gate_bf16_vec_kernel(bf16_t* __restrict__ a, const bf16_
     }
 }
 
-extern "C" int ia_sigmoid_gate(void* a, const void* g, int rows, int cols, int g_ld, int g_off, int dtype, hipStream_t stream) {
-    IA_CHECK(rows >= 0 && cols > 0 && g_off >= 0 && g_off + cols <= g_ld, "sigmoid_gate: rows=%d cols=%d pitch=%d offset=%d", rows,
-             cols, g_ld, g_off);
+// group: columns that share one gate value (1: a value a column; a head's width: a value a head)
+extern "C" int ia_sigmoid_gate(void* a, const void* g, int rows, int cols, int g_ld, int g_off, int group, int dtype,
+                               hipStream_t stream) {
+    IA_CHECK(rows >= 0 && cols > 0 && group >= 1 && cols % group == 0 && g_off >= 0 && g_off + cols / group <= g_ld,
+             "sigmoid_gate: rows=%d cols=%d pitch=%d offset=%d group=%d", rows, cols, g_ld, g_off, group);
     if (rows == 0) return 0;
     const size_t total = (size_t)rows * cols;
     const int block = 256;
-    if (dtype == IA_BF16 && cols % 8 == 0 && g_ld % 8 == 0 && g_off % 8 == 0 && ((((uintptr_t)a) | ((uintptr_t)g)) & 15) == 0) {
+    if (group == 1 && dtype == IA_BF16 && cols % 8 == 0 && g_ld % 8 == 0 && g_off % 8 == 0 && ((((uintptr_t)a) | ((uintptr_t)g)) & 15) == 0) {
         const size_t vecs = total / 8;
         const size_t want = (vecs + block - 1) / block;
         sigmoid_gate_bf16_vec_kernel<<<(unsigned)(want < 65535 * 8 ? want : 65535 * 8), block, 0, stream>>>(
@@ -297,9 +300,9 @@ extern "C" int ia_sigmoid_gate(void* a, const void* g, int rows, int cols, int g
     const size_t want = (total + block - 1) / block;
     const int grid = (int)(want < 65535 ? want : 65535);
     if (dtype == IA_F32)
-        sigmoid_gate_kernel<float><<<grid, block, 0, stream>>>((float*)a, (const float*)g, cols, g_ld, g_off, total);
+        sigmoid_gate_kernel<float><<<grid, block, 0, stream>>>((float*)a, (const float*)g, cols, g_ld, g_off, group, total);
     else if (dtype == IA_BF16)
-        sigmoid_gate_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)a, (const bf16_t*)g, cols, g_ld, g_off, total);
+        sigmoid_gate_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)a, (const bf16_t*)g, cols, g_ld, g_off, group, total);
     else
         IA_CHECK(false, "sigmoid_gate: unknown dtype %d", dtype);
     IA_LAUNCH_CHECK("sigmoid_gate");

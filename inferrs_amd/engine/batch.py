@@ -52,6 +52,8 @@ class StepContext:
     stream_norm: Any = None                 # and the norm part that will read the stream next
     partial_sums: bool = False              # set by a block whose norms take a part's last product split along k
     pass_input: Any = None                  # set by the model before a stop that begins a pass of a looped range: (rows or None, vector); the block takes it
+    side_rows: Any = None                   # the rows of an embedding's second table for the step's tokens, which layers take slices of
+    normed: Any = None                      # (norm part, rows): the stream's rows through that norm already, left by the block before
     post_rows: Any = None                   # a 32-bit stream's rows once more in the products' precision, where a part has them already (the embedding, a block's last kernel)
     _tables: Dict[Any, Any] = field(default_factory=dict)
 

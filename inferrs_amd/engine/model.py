@@ -11,6 +11,7 @@ from .. import ops
 from ..config.spec import ModelSpec, SpecError
 from ..parts.base import block_class, part_class
 from ..parts.linear import Linear
+from ..parts.norm import build_norm
 from .batch import StepContext
 
 DTYPES = {"float32": torch.float32, "f32": torch.float32, "fp32": torch.float32,
@@ -52,8 +53,7 @@ class DecoderModel:
             self.pass_input = pass_cls(spec.pass_input, take(pass_cls.tensors(spec.pass_input)), dtype, device)
         self.final_norm = None
         if spec.final_norm is not None:
-            self.final_norm = part_class("norm", spec.final_norm)(
-                spec.final_norm, {"weight": tensors.pop(spec.final_norm_name)}, dtype, device)
+            self.final_norm = build_norm(spec.final_norm_name, spec.final_norm, tensors, dtype, device, pop=True)
 
     @property
     def graph_safe(self) -> bool:

@@ -399,15 +399,19 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, page_si
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
                       *, window: Optional[int], scale: float, max_kv_len: Optional[int] = None,
-                      split: Optional[bool] = None, sink: bool = False) -> torch.Tensor:
+                      split: Optional[bool] = None, sink: bool = False, mask_chunk: Optional[int] = None,
+                      sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [n, nq, d] against the paged cache (values may have a width of their own: v_cache [pages, nkv, dv, page_size],
     the result is [n, nq, dv]); token i sees the keys at positions <= positions[i]
     (and > positions[i] - window) of row token_seq[i] of the table.  Any head size up to 512, any
     page size, 32-bit or bfloat16 storage, all arithmetic in 32-bit.  `max_kv_len`: an upper bound of
     positions + 1 (default: what the table can hold).  Steps of few tokens run a wave a segment of 512 keys
     and a merge kernel (`split`; None: the kernel's own rule); the bits are the same either way.
-    `sink`: the softmax's denominator holds one more term, exp(0): a key of score 0 that has no value."""
-    _dev(q, k_cache, v_cache, positions, token_seq, block_table)
+    `sink`: the softmax's denominator holds one more term, exp(0): a key of score 0 that has no value; `sinks` [nq]
+    (32-bit): the term is exp(sinks[h]) for query head h instead (not scaled).  `mask_chunk`: a token sees the keys of its
+    own chunk of that many positions only (chunks counted from position 0 of the sequence), up to itself."""
+    _dev(q, k_cache, v_cache, positions, token_seq, block_table, sinks)
+    sink = _check_sinks(sinks, sink, q.shape[1])
     _i32(positions, "positions"); _i32(token_seq, "token_seq"); _i32(block_table, "block_table")
     n, nq, d = q.shape
     nkv, page_size = k_cache.shape[1], k_cache.shape[2]
@@ -426,8 +430,17 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _check(lib.ia_attention_generic(
         _p(out), _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_seq), _p(block_table), n,
         block_table.shape[1], nq, nkv, d, dv, page_size, int(window or 0), ctypes.c_float(scale), _dt(q),
-        _p(ws), max_kv_len, int(bool(sink)), _stream()))
+        _p(ws), max_kv_len, int(bool(sink)), int(mask_chunk or 0), _p(sinks), _stream()))
     return out
+
+
+def _check_sinks(sinks: Optional[torch.Tensor], sink: bool, nq: int) -> bool:
+    if sinks is None:
+        return bool(sink)
+    _f32(sinks, "sinks")
+    if sinks.numel() != nq or not sinks.is_contiguous():
+        raise KernelError(f"attention: {sinks.numel()} sink values for {nq} query heads")
+    return True
 
 
 ATTN_TARGET_WAVES = 2048       # waves wanted in flight before the keys stop being split
@@ -505,14 +518,16 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                    cu_tokens: torch.Tensor, block_table: torch.Tensor, *, max_q_len: int, max_kv_len: int,
                    window: Optional[int], scale: float, splits: Optional[int] = None,
                    seqs: Optional[Tuple[int, int]] = None, tokens: Optional[Tuple[int, int]] = None,
-                   out: Optional[torch.Tensor] = None, sink: bool = False) -> torch.Tensor:
+                   out: Optional[torch.Tensor] = None, sink: bool = False, mask_chunk: Optional[int] = None,
+                   sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The matrix-core kernel: bfloat16, head sizes in steps of 16 up to 256, page sizes in steps
     of 16.  Request s owns tokens cu_tokens[s]..cu_tokens[s+1] at consecutive positions.  `seqs` =
     (first, count) and `tokens` = (first, count) restrict the call to a run of requests and their
     tokens (the whole step by default); `max_q_len` and `max_kv_len` are the largest token count of
     one of these requests in this step and their largest length after it.  `out` receives the result
-    (rows outside `tokens` are left alone)."""
-    _dev(q, k_cache, v_cache, positions, cu_tokens, block_table, out)
+    (rows outside `tokens` are left alone).  `sink`, `sinks`, `mask_chunk`: as in `attention_generic`."""
+    _dev(q, k_cache, v_cache, positions, cu_tokens, block_table, out, sinks)
+    sink = _check_sinks(sinks, sink, q.shape[1])
     _i32(positions, "positions"); _i32(cu_tokens, "cu_tokens"); _i32(block_table, "block_table")
     n, nq, d = q.shape
     nkv, page_size = k_cache.shape[1], k_cache.shape[2]
@@ -549,7 +564,8 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     _check(lib.ia_attention_mfma(
         _p(out), _p(ws), _p(q), _p(k_cache), _p(v_cache), _p(block_table), _p(cu_tokens), _p(positions),
         n, seq_begin, n_seqs, token_begin, n_tokens, max_q_len, max_kv_len, block_table.shape[1], nq, nkv, d,
-        page_size, int(window or 0), ctypes.c_float(scale), splits, chunk, int(bool(sink)), _stream()), target)
+        page_size, int(window or 0), ctypes.c_float(scale), splits, chunk, int(bool(sink)), int(mask_chunk or 0), _p(sinks),
+        _stream()), target)
     return out
 
 
@@ -1231,8 +1247,8 @@ def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
 
 
 # ---- several residual streams, latent attention, gated recurrence, routed experts -----------------
-from .mix import (clamped_gate_mul, conv_step, embed_gather_scaled, experts_forward, head_product,    # noqa: E402
-                  latent_prep, postnorm_step, rglru_scan, route, scale_inplace, sigmoid_gate, softcap,
+from .mix import (clamped_gate_mul, conv_step, embed_gather_scaled, experts_forward, gate_rows, head_product,    # noqa: E402
+                  latent_prep, parallel_step, postnorm_step, rglru_scan, route, scale_inplace, sigmoid_gate, softcap,
                   streams_open, streams_step)
 from .state import (activation, conv_act_step, exp_gates, group_norm_gate, linear_scan, sandwich_step,   # noqa: E402
                     step_gates)

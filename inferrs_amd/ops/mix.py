@@ -91,14 +91,18 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
 def latent_prep(proj: torch.Tensor, *, heads: int, dim: int, rot_dim: int, rank: int, rotated: int, q_off: int,
                 down_off: int, norm_weight: torch.Tensor, eps: float, cos: Optional[torch.Tensor],
                 sin: Optional[torch.Tensor], magnitude: float, k_cache: Optional[torch.Tensor],
-                v_cache: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_size: int) -> torch.Tensor:
+                v_cache: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_size: int,
+                interleaved: bool = False, q_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """From the projections' rows to the attention's operands: the latent row is normed (32-bit) and written, with
     the rotated shared key part behind it, to the key cache as a row and to the value cache as a column; returns
     q [n, heads, rank + rot_dim] with the rotated parts in place at [rank:], the first `rank` features left for
-    `head_product` to fill."""
-    _dev(proj, norm_weight, cos, sin, k_cache, v_cache, slots)
+    `head_product` to fill.  `interleaved`: of the rotated features 2i turns with 2i + 1 (else i with i + rotated / 2).
+    `q_rows` [n, ...]: the queries' rows where they are no part of `proj` (a product of their own), q at `q_off` there."""
+    _dev(proj, norm_weight, cos, sin, k_cache, v_cache, slots, q_rows)
     _f32(norm_weight, "norm weight"); _f32(cos, "cos"); _f32(sin, "sin")
     n, ld = proj.shape
+    if q_rows is not None and (q_rows.dim() != 2 or q_rows.shape[0] != n or q_rows.dtype != proj.dtype or q_rows.stride(1) != 1):
+        raise KernelError(f"latent_prep: the queries' rows {tuple(q_rows.shape)} {q_rows.dtype} do not fit {n} rows of {proj.dtype}")
     D = rank + rot_dim
     if norm_weight.numel() != rank:
         raise KernelError(f"latent_prep: the norm weight has {norm_weight.numel()} entries, the rank is {rank}")
@@ -117,17 +121,19 @@ def latent_prep(proj: torch.Tensor, *, heads: int, dim: int, rot_dim: int, rank:
     _check(library().ia_latent_prep(
         _p(q), _p(k_cache if slots is not None else None), _p(v_cache if slots is not None else None), _p(proj),
         _p(norm_weight), _p(cos), _p(sin), _p(slots), n, heads, dim, rot_dim, rank, rotated, q_off, down_off, ld,
-        page_size, ctypes.c_float(eps), ctypes.c_float(magnitude), _dt(proj), _stream()))
+        page_size, ctypes.c_float(eps), ctypes.c_float(magnitude), int(bool(interleaved)), _p(q_rows),
+        q_rows.stride(0) if q_rows is not None else 0, _dt(proj), _stream()))
     return q
 
 
 def head_product(x: torch.Tensor, w: torch.Tensor, *, x_off: int = 0, x_head: Optional[int] = None,
                  out: Optional[torch.Tensor] = None, o_off: int = 0, o_head: Optional[int] = None,
                  out_dtype: Optional[torch.dtype] = None, gate: Optional[torch.Tensor] = None,
-                 g_off: int = 0) -> torch.Tensor:
+                 g_off: int = 0, gate_per_head: bool = False) -> torch.Tensor:
     """A product with a matrix of its own for every head: w [H, n_out, k_in]; x is 2-D, head h of row t starts at
     x[t, x_off + h * x_head] (x_head default k_in); the result goes to out[t, o_off + h * o_head ...] (a new
-    [n, H * n_out] tensor by default).  `gate` (2-D, head h at g_off + h * n_out): times its sigmoid."""
+    [n, H * n_out] tensor by default).  `gate` (2-D, head h at g_off + h * n_out): times its sigmoid; `gate_per_head`: one
+    gate value a head, head h's at g_off + h."""
     _dev(x, w, out, gate)
     H, n_out, k_in = w.shape
     n, x_ld = x.shape
@@ -141,7 +147,7 @@ def head_product(x: torch.Tensor, w: torch.Tensor, *, x_off: int = 0, x_head: Op
         raise KernelError("head_product: the gate must be 2-D rows of x's precision")
     _check(library().ia_head_product(
         _p(out), _p(x), _p(w), _p(gate), n, H, n_out, k_in, x_ld, x_off, x_head, out.shape[1], o_off, o_head,
-        gate.shape[1] if gate is not None else 0, g_off, _dt(x), _dt(w), _dt(out), _stream()))
+        gate.shape[1] if gate is not None else 0, g_off, int(bool(gate_per_head)), _dt(x), _dt(w), _dt(out), _stream()))
     return out
 
 
@@ -205,25 +211,30 @@ def rglru_scan(u: torch.Tensor, z: torch.Tensor, proj: torch.Tensor, *, branch_o
 # ---- routed experts -----------------------------------------------------------------------------
 
 def route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, score: str = "sigmoid",
-          renormalize: bool = False, choice_bias: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+          renormalize: bool = False, choice_bias: Optional[torch.Tensor] = None, gates: int = 0):
     """Router logits in 32-bit (router [E, width] in the precision of h; every logit is a sum of 32-bit
     multiply-adds in an order that the width alone decides), the `top` experts by score for every row:
     (experts int32 [n, top] best first, weights float32 [n, top] = score * scale).  `choice_bias` [E] (32-bit):
-    the choice goes by score + bias, the weights stay the scores."""
+    the choice goes by score + bias, the weights stay the scores.  `gates`: the last `gates` rows of `router` are no
+    experts: they take no part in the choice, and the sigmoids of their logits (formed like the others, in 32-bit) come
+    back as a third result, float32 [n, gates]."""
     _dev(h, router, choice_bias); _f32(choice_bias, "choice_bias")
-    if choice_bias is not None and choice_bias.numel() != router.shape[0]:
-        raise KernelError(f"route: {choice_bias.numel()} biases for {router.shape[0]} outputs of the router")
     n, W = h.shape
-    E = router.shape[0]
-    if (router.shape[1] != W or router.dtype != h.dtype or not (1 <= top <= min(E, MAX_TOP)) or E > MAX_EXPERTS
+    E = router.shape[0] - gates
+    if gates < 0 or E < 1:
+        raise KernelError(f"route: {gates} gate rows in a router of {router.shape[0]} rows")
+    if choice_bias is not None and choice_bias.numel() != E:
+        raise KernelError(f"route: {choice_bias.numel()} biases for {E} outputs of the router")
+    if (router.shape[1] != W or router.dtype != h.dtype or not (1 <= top <= min(E, MAX_TOP)) or E + gates > MAX_EXPERTS
             or score not in SCORE_FUNCTIONS):
         raise KernelError(f"route: router {tuple(router.shape)} {router.dtype}, top {top}, score {score!r} (up to {MAX_EXPERTS} "
                           f"experts, top up to {MAX_TOP}, scores {sorted(SCORE_FUNCTIONS)})")
     sel = torch.empty((n, top), dtype=torch.int32, device=h.device)
     weight = torch.empty((n, top), dtype=torch.float32, device=h.device)
+    gate_out = torch.empty((n, gates), dtype=torch.float32, device=h.device) if gates else None
     _check(library().ia_route(_p(sel), _p(weight), _p(h), _p(router), n, W, E, top, ctypes.c_float(scale),
-                              SCORE_FUNCTIONS[score], int(renormalize), _p(choice_bias), _dt(h), _stream()))
-    return sel, weight
+                              SCORE_FUNCTIONS[score], int(renormalize), _p(choice_bias), gates, _p(gate_out), _dt(h), _stream()))
+    return (sel, weight, gate_out) if gates else (sel, weight)
 
 
 def tile_weights(w: torch.Tensor) -> torch.Tensor:
@@ -242,13 +253,17 @@ def experts_tiled_fits(dtype: torch.dtype, width: int, ff: int) -> bool:
 
 
 def experts_forward(h: torch.Tensor, sel: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
-                    limit: float, alpha: float, ff: Optional[int] = None) -> torch.Tensor:
+                    limit: float, alpha: float, ff: Optional[int] = None, in_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The chosen experts of every row: w_gate_up [E, 2 ff, width] (gate rows, then up rows), w_down [E, width, ff],
     or both as tiles (`tile_weights` of [E, 2, ff, width] and of [E, width, ff]; then `ff` is given);
     act = g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).  Returns one
     32-bit output row a (row, k) pair, [n, top, width]; nothing is added up here.  A choice of E or beyond names no
-    expert with weights: its row is left unwritten (whoever adds the rows up knows what stands for it)."""
-    _dev(h, sel, w_gate_up, w_down); _i32(sel, "sel")
+    expert with weights: its row is left unwritten (whoever adds the rows up knows what stands for it).  `in_weight`
+    [n, top] (32-bit): pair (row, k) runs its expert on in_weight[row, k] * h[row] (the factor meets the two products'
+    32-bit sums ahead of the limits, which is the same number)."""
+    _dev(h, sel, w_gate_up, w_down, in_weight); _i32(sel, "sel"); _f32(in_weight, "in_weight")
+    if in_weight is not None and (tuple(in_weight.shape) != tuple(sel.shape) or not in_weight.is_contiguous()):
+        raise KernelError(f"experts: input weights {tuple(in_weight.shape)} for choices {tuple(sel.shape)}")
     n, W = h.shape
     top = sel.shape[1]
     tiled = w_gate_up.dim() == 6
@@ -279,7 +294,7 @@ def experts_forward(h: torch.Tensor, sel: torch.Tensor, w_gate_up: torch.Tensor,
     act = torch.empty((pairs, ff), dtype=h.dtype, device=h.device)
     _check(lib.ia_experts_gate_up(_p(act), _p(h), _p(w_gate_up), _p(order), _p(t_exp), _p(t_first), _p(t_rows), _p(meta),
                                   pairs, E, top, W, ff, ctypes.c_float(limit), ctypes.c_float(alpha), tile, int(tiled),
-                                  _dt(h), _stream()))
+                                  _p(in_weight), _dt(h), _stream()))
     y = torch.empty((n, top, W), dtype=torch.float32, device=h.device)
     _check(lib.ia_experts_down(_p(y), _p(act), _p(w_down), _p(order), _p(t_exp), _p(t_first), _p(t_rows), _p(meta), pairs,
                                E, W, ff, tile, int(tiled), _dt(h), _stream()))
@@ -359,13 +374,15 @@ def embed_gather_scaled(table: torch.Tensor, ids: torch.Tensor, scale: float, ro
     return (out, lo) if rounded else out
 
 
-def sigmoid_gate(a: torch.Tensor, g: torch.Tensor, g_off: int = 0) -> torch.Tensor:
-    """a[:, c] *= sigmoid(g[:, g_off + c]) in place; a [n, cols] contiguous, g 2-D rows of the same precision."""
+def sigmoid_gate(a: torch.Tensor, g: torch.Tensor, g_off: int = 0, group: int = 1) -> torch.Tensor:
+    """a[:, c] *= sigmoid(g[:, g_off + c // group]) in place; a [n, cols] contiguous, g 2-D rows of the same precision.
+    `group`: neighbouring columns that share one gate value (a head's width: one value a head)."""
     _dev(a, g)
     n, cols = a.shape
-    if g.dim() != 2 or g.shape[0] != n or g.dtype != a.dtype or g_off < 0 or g_off + cols > g.shape[1] or not a.is_contiguous():
+    if (g.dim() != 2 or g.shape[0] != n or g.dtype != a.dtype or g_off < 0 or group < 1 or cols % group
+            or g_off + cols // group > g.shape[1] or not a.is_contiguous()):
         raise KernelError(f"sigmoid_gate: a gate {tuple(g.shape)} {g.dtype} at {g_off} does not fit rows {tuple(a.shape)} {a.dtype}")
-    _check(library().ia_sigmoid_gate(_p(a), _p(g), n, cols, g.stride(0), g_off, _dt(a), _stream()))
+    _check(library().ia_sigmoid_gate(_p(a), _p(g), n, cols, g.stride(0), g_off, group, _dt(a), _stream()))
     return a
 
 
@@ -386,3 +403,91 @@ def scale_inplace(x: torch.Tensor, factor: float) -> torch.Tensor:
     _dev(x); _f32(x, "x")
     _check(library().ia_scale(_p(x), ctypes.c_longlong(x.numel()), ctypes.c_float(factor), _stream()))
     return x
+
+
+# ---- a stream whose sub-layers read one normed copy ---------------------------------------------------------------------
+
+def parallel_step(x: torch.Tensor, *, y1=None, y2=None, y3=None, y3_scale: Optional[torch.Tensor] = None,
+                  routed: Optional[torch.Tensor] = None, routed_weights: Optional[torch.Tensor] = None,
+                  enter: Optional[torch.Tensor] = None, enter_weight: Optional[torch.Tensor] = None, enter_eps: float = 0.0,
+                  x_dtype: Optional[torch.dtype] = None, norm_weight: Optional[torch.Tensor] = None,
+                  norm_bias: Optional[torch.Tensor] = None, norm_eps: float = 0.0, center: bool = True,
+                  h_dtype: Optional[torch.dtype] = None, rows: Optional[torch.Tensor] = None):
+    """What stands between two layers around a 32-bit stream x [n, width] (changed in place) whose sub-layers all read
+    one normed copy of it:
+
+        x <- x + y1 + y2 + sum_k [routed_weights[:, k]] routed[:, k] + y3_scale[:, None] * y3
+        x <- x + rmsnorm(enter) * enter_weight                       (`enter_eps` inside the root)
+        h  = (x - mean) / sqrt(var + norm_eps) * norm_weight + norm_bias   (`center` False: an RMS norm; the bias may be None)
+
+    Every line and every addend may be absent.  y1, y2, y3 may each be a product still split along its k (`Partials`).
+    Returns (the new x once more in `x_dtype` or None, h in `h_dtype` or None).  `rows` (int32): only these rows go
+    through the norm; nothing is added and the stream is left as it is."""
+    from . import Partials
+    ys = [y1, y2, y3]
+    dense = [t for t in ys + [enter] if t is not None]
+    if any(isinstance(t, Partials) for t in dense) and any(not isinstance(t, Partials) and t.dtype != torch.float32 for t in dense):
+        ys = [t.materialize() if isinstance(t, Partials) else t for t in ys]       # (one precision for all)
+    splits = [1, 1, 1]
+    for i, t in enumerate(ys):
+        if isinstance(t, Partials):
+            splits[i], ys[i] = t.parts.shape[0], t.parts
+    y1, y2, y3 = ys
+    _dev(x, y1, y2, y3, y3_scale, routed, routed_weights, enter, enter_weight, norm_weight, norm_bias, rows)
+    for t, name in ((x, "the stream"), (y3_scale, "y3_scale"), (routed, "routed rows"), (routed_weights, "routed weights"),
+                    (enter_weight, "enter_weight"), (norm_weight, "norm weight"), (norm_bias, "norm bias")):
+        _f32(t, name)
+    n, W = x.shape
+    given = [t for t in (y1, y2, y3, enter) if t is not None]
+    for t, sp in ((y1, splits[0]), (y2, splits[1]), (y3, splits[2]), (enter, 1)):
+        if t is None:
+            continue
+        if (tuple(t.shape[-2:]) != (n, W) or t.dtype != given[0].dtype or not t.is_contiguous() or t.dim() not in (2, 3)
+                or (t.dim() == 3 and (t.shape[0] != sp or t.dtype != torch.float32))):
+            raise KernelError(f"parallel_step: an output {tuple(t.shape)} {t.dtype} does not fit the stream [{n}, {W}]")
+    top = 0
+    if routed is not None:
+        top = routed.shape[1]
+        if (routed.dim() != 3 or tuple(routed.shape) != (n, top, W) or top > MAX_TOP or not routed.is_contiguous()
+                or (routed_weights is not None and tuple(routed_weights.shape) != (n, top))):
+            raise KernelError(f"parallel_step: routed rows {tuple(routed.shape)} do not fit [{n}, top <= {MAX_TOP}, {W}]")
+    if y3_scale is not None and (y3 is None or y3_scale.numel() != n):
+        raise KernelError("parallel_step: a factor a row goes with y3 and has one entry a row")
+    if enter is not None and (enter_weight is None or enter_weight.numel() != W):
+        raise KernelError("parallel_step: a row that enters comes with its norm's weight")
+    for t in (norm_weight, norm_bias):
+        if t is not None and t.numel() != W:
+            raise KernelError(f"parallel_step: the norm has {t.numel()} entries, the stream is {W} wide")
+    if h_dtype is not None and norm_weight is None:
+        raise KernelError("parallel_step: normed rows come with the norm's weight")
+    count = n
+    if rows is not None:
+        _i32(rows, "rows")
+        count = rows.numel()
+        if h_dtype is None or given or routed is not None or x_dtype is not None:
+            raise KernelError("parallel_step: a row list goes with normed rows out and nothing to add")
+    out_dtype = h_dtype if h_dtype is not None else x_dtype
+    if h_dtype is not None and x_dtype is not None and h_dtype != x_dtype:
+        raise KernelError("parallel_step: one precision for both outputs")
+    xr = torch.empty((n, W), dtype=x_dtype, device=x.device) if x_dtype is not None else None
+    h = torch.empty((count, W), dtype=h_dtype, device=x.device) if h_dtype is not None else None
+    _check(library().ia_parallel_step(
+        _p(x), _p(y1), _p(y2), _p(y3), splits[0], splits[1], splits[2], _p(y3_scale), _p(routed), _p(routed_weights), top,
+        _p(enter), _p(enter_weight), ctypes.c_float(enter_eps), _p(xr), _p(norm_weight), _p(norm_bias),
+        ctypes.c_float(norm_eps), int(bool(center)), _p(h), _p(rows), count, W, _dt(given[0]) if given else 0,
+        _DT[out_dtype] if out_dtype is not None else 0, _stream()))
+    return xr, h
+
+
+def gate_rows(g: torch.Tensor, e: torch.Tensor, e_off: int, activation: str = "gelu_tanh") -> torch.Tensor:
+    """act(g) * e[:, e_off : e_off + cols] for rows g [n, cols] (contiguous) and wider rows e of the same precision."""
+    from . import activation_code
+    _dev(g, e)
+    n, cols = g.shape
+    if (e.dim() != 2 or e.shape[0] != n or e.dtype != g.dtype or e_off < 0 or e_off + cols > e.shape[1] or e.stride(1) != 1
+            or not g.is_contiguous()):
+        raise KernelError(f"gate_rows: rows {tuple(e.shape)} {e.dtype} at {e_off} do not fit gates {tuple(g.shape)} {g.dtype}")
+    out = torch.empty_like(g)
+    _check(library().ia_gate_rows(_p(out), _p(g), _p(e), n, cols, e.stride(0), e_off, activation_code(activation), _dt(g),
+                                  _stream()))
+    return out

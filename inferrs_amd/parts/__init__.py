@@ -2,7 +2,7 @@ from .base import (BlockBase, Embedding, FeedForward, FixedState, Head, Mixer, N
                    block_class, part_class, register_block, register_embedding, register_ffn, register_head,
                    register_mixer, register_norm, register_pass_input, register_position)
 from . import (norm, position, mlp, attention, io, block, latent_attention, recurrence, experts, streams,   # registers the built-in parts
-               sandwich, matrix_state, postnorm)
+               sandwich, matrix_state, postnorm, parallel)
 from .assemble import generated_tensors, layer_tensors, model_tensors
 from .block import Block
 from .linear import Linear

@@ -6,6 +6,7 @@ from typing import Dict, Set, Tuple
 from ..config.spec import ModelSpec
 from ..weights.loader import TensorSpec
 from .base import block_class, part_class
+from .norm import norm_tensors
 
 
 def layer_tensors(layer) -> Dict[str, TensorSpec]:
@@ -18,8 +19,7 @@ def model_tensors(spec: ModelSpec) -> Tuple[Dict[str, TensorSpec], Set[str]]:
     for layer in spec.layers:
         expected.update(layer_tensors(layer))
     if spec.final_norm is not None:
-        (ts,) = part_class("norm", spec.final_norm).tensors(spec.final_norm).values()
-        expected[spec.final_norm_name] = ts
+        expected.update(norm_tensors(spec.final_norm_name, spec.final_norm))
     head = part_class("head", spec.head)
     expected.update(head.tensors(spec.head))
     if getattr(spec, "pass_input", None) is not None:

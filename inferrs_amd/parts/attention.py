@@ -15,7 +15,11 @@ their own (`v_head_dim`: the cache's value array, the heads' outputs and the out
 sigmoid gate on the joined heads (`gate`: sigmoid(W_g h), one product with the projections), and a layer without keys and
 values of its own (`own_kv` False: its stop of the schedule reads another stop's cache, after that layer's norm and
 rotation, with its own queries, window and scale).  Such a layer's rows are [q | k | v | g], whatever of these it has, and
-go through the kernels that take rows of any layout.
+go through the kernels that take rows of any layout.  Further still: a mask of chunks instead of a window (`mask_chunk`:
+a query sees the keys of its own chunk of that many positions, up to itself; every attention kernel takes it beside the
+window), one gate value a head instead of one a feature (`gate_per_head`), and q and k at unit root mean square a head
+without a learned weight (`qk_unit_norm`: the norm kernels run with a weight of ones; a turn by position keeps a head's
+sum of squares, so it does not matter on which side of the turn the norm stands).
 """
 from __future__ import annotations
 
@@ -56,8 +60,8 @@ class Attention(Mixer):
             "o_proj.weight": TensorSpec((spec.hidden, spec.n_heads * spec.value_dim)),
         }
         if spec.gate:
-            t["g_proj.weight"] = TensorSpec((spec.n_heads * spec.value_dim, spec.hidden))
-        if spec.qk_norm is not None:
+            t["g_proj.weight"] = TensorSpec((spec.n_heads * (1 if spec.gate_per_head else spec.value_dim), spec.hidden))
+        if spec.qk_norm is not None and not spec.qk_unit_norm:
             t["q_norm.weight"] = TensorSpec((spec.head_dim,), "norm")
             t["k_norm.weight"] = TensorSpec((spec.head_dim,), "norm")
         if spec.qkv_bias:
@@ -87,6 +91,10 @@ class Attention(Mixer):
             raise SpecError(f"attention: the rotated part of a head ({rot}) must be even and within head_dim {spec.head_dim}")
         if spec.window is not None and spec.window < 1:
             raise SpecError(f"attention: window {spec.window} must be >= 1")
+        if spec.mask_chunk is not None and spec.mask_chunk < 1:
+            raise SpecError(f"attention: mask_chunk {spec.mask_chunk} must be >= 1")
+        if spec.qk_unit_norm and spec.qk_norm is None:
+            raise SpecError("attention: qk_unit_norm takes size and eps from qk_norm")
         if spec.qk_norm is not None and spec.qk_norm.size != spec.head_dim:
             raise SpecError("attention: qk_norm must span head_dim")
         if not (1 <= spec.value_dim <= 512):
@@ -98,10 +106,9 @@ class Attention(Mixer):
         tensors = {k: tensors[named.get(k, k)] for k in self._tensors(spec) if named.get(k, k) in tensors}
         # rows of the plain layout [q | k | v], heads of one width, go through the kernels made for it; everything else
         # (a gate in the rows, values of another width, no keys at all) through those that take any layout
-        self.plain = spec.own_kv and not spec.gate and spec.value_dim == spec.head_dim
+        self.plain = (spec.own_kv and not spec.gate and spec.value_dim == spec.head_dim and not spec.mask_chunk
+                      and not spec.qk_unit_norm)
         if not self.plain:
-            if spec.qkv_bias:
-                raise SpecError("attention: biases go with rows of the plain layout [q | k | v]")
             self._init_general(spec, tensors, dtype, device)
             return
         if spec.values_from_keys:
@@ -125,18 +132,27 @@ class Attention(Mixer):
     def _init_general(self, spec: AttentionSpec, tensors, dtype, device):
         H, G, d, dv = spec.n_heads, spec.n_kv_heads, spec.head_dim, spec.value_dim
         stacked, at = [tensors["q_proj.weight"]], H * d
+        biases = [tensors["q_proj.bias"]] if spec.qkv_bias else None
         self.q_off, self.k_off, self.v_off, self.g_off = 0, None, None, None
         if spec.own_kv:
             stacked += [tensors["k_proj.weight"], tensors["v_proj.weight"]]
+            if spec.qkv_bias:
+                biases += [tensors["k_proj.bias"], tensors["v_proj.bias"]]
             self.k_off, self.v_off, at = at, at + G * d, at + G * d + G * dv
         if spec.gate:
             stacked.append(tensors["g_proj.weight"])
-            self.g_off, at = at, at + H * dv
-        self.qkv = Linear(stacked, dtype, device)
+            g_rows = H * (1 if spec.gate_per_head else dv)
+            if spec.qkv_bias:                        # (the gate has no bias: zeros keep the one fused product)
+                biases.append(torch.zeros((g_rows,), dtype=tensors["q_proj.bias"].dtype))
+            self.g_off, at = at, at + g_rows
+        self.qkv = Linear(stacked, dtype, device, biases)
         self.o = Linear([tensors["o_proj.weight"]], dtype, device, [tensors["o_proj.bias"]] if spec.o_bias else None)
         self.q_norm_w = self.k_norm_w = None
         self.norm_eps, self.norm_add_one = 0.0, False
-        if spec.qk_norm is not None:
+        if spec.qk_unit_norm:
+            self.q_norm_w = self.k_norm_w = torch.ones((d,), dtype=torch.float32, device=device)
+            self.norm_eps = float(spec.qk_norm.eps)
+        elif spec.qk_norm is not None:
             self.q_norm_w = tensors["q_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
             if spec.own_kv:
                 self.k_norm_w = tensors["k_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
@@ -163,14 +179,14 @@ class Attention(Mixer):
         a = self._attend(ctx, q, cache, group)
         joined = a.view(a.shape[0], H * dv)
         if s.gate:
-            ops.sigmoid_gate(joined, proj, self.g_off)
+            ops.sigmoid_gate(joined, proj, self.g_off, group=dv if s.gate_per_head else 1)
         return self._project(ctx, joined)
 
     def _attend(self, ctx, q, cache, group):
         """The paged attention of the step's queries: the matrix cores where they take the sizes, else the plain kernel."""
         s = self.spec
         if ops.attention_mfma_fits(q.dtype, s.head_dim, group.page_size, s.value_dim):
-            common = dict(window=s.window, scale=s.softmax_scale, sink=s.sink)
+            common = dict(window=s.window, scale=s.softmax_scale, sink=s.sink, mask_chunk=s.mask_chunk)
             if 0 < ctx.n_single < ctx.n_seqs:
                 # single tokens (decode) and portions of prompts want different launches: the first
                 # split their long key ranges between waves, the second have columns enough
@@ -185,7 +201,8 @@ class Attention(Mixer):
             return ops.attention_mfma(q, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table,
                                       max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len, **common)
         return ops.attention_generic(q, cache.k, cache.v, ctx.positions, ctx.token_seq, group.block_table,
-                                     window=s.window, scale=s.softmax_scale, max_kv_len=ctx.max_kv_len, sink=s.sink)
+                                     window=s.window, scale=s.softmax_scale, max_kv_len=ctx.max_kv_len, sink=s.sink,
+                                     mask_chunk=s.mask_chunk)
 
     def load_notes(self, page_size: int):
         """What the log should say once when a model with this part is set up: a decode step that cannot take the

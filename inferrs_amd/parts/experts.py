@@ -10,7 +10,10 @@ this).
 Options of the spec: `identity` more outputs of the router behind the experts', each standing for an expert that hands
 its input on (no tensors: `RoutedRows.sel` and `.real_experts` tell whoever adds the rows up which pairs these are, and
 the stream's own row takes their place); `correction`, a vector added to the scores for the choice only; `shared`, a
-feed-forward of the experts' form that runs for every token (`ClampedMlp`; its output rides along as `RoutedRows.extra`)."""
+feed-forward of the experts' form that runs for every token (`ClampedMlp`; its output rides along as `RoutedRows.extra`),
+behind a sigmoid gate a token with `shared_gate` (its row stands behind the router's in one matrix, so that the gate is
+formed like a router's logit: `RoutedRows.extra_scale`); `weight_on_input`, a chosen expert runs on weight * h and its
+output counts as it is (`RoutedRows.weights` is None then)."""
 from __future__ import annotations
 
 from typing import Dict
@@ -27,14 +30,16 @@ from .linear import Linear, to_compute
 class RoutedRows:
     """rows [n, top, width] (32-bit) and weights [n, top] (32-bit): the output is sum_k weights[:, k] * rows[:, k].
     `sel` [n, top] with `real_experts`: a pair whose choice is `real_experts` or more has no row here; the
-    feed-forward's own input stands for it.  `extra` [n, width]: a dense output to be added beside the rows."""
-    __slots__ = ("rows", "weights", "sel", "real_experts", "extra")
+    feed-forward's own input stands for it.  `extra` [n, width]: a dense output to be added beside the rows, times
+    `extra_scale` [n] (32-bit) where that is given.  `weights` None: the rows are added as they are."""
+    __slots__ = ("rows", "weights", "sel", "real_experts", "extra", "extra_scale")
 
-    def __init__(self, rows: torch.Tensor, weights: torch.Tensor, sel=None, real_experts: int = 0, extra=None):
+    def __init__(self, rows: torch.Tensor, weights, sel=None, real_experts: int = 0, extra=None, extra_scale=None):
         self.rows, self.weights, self.sel, self.real_experts, self.extra = rows, weights, sel, real_experts, extra
+        self.extra_scale = extra_scale
 
     def materialize(self) -> torch.Tensor:
-        if self.sel is not None or self.extra is not None:
+        if self.sel is not None or self.extra is not None or self.weights is None:
             raise SpecError("routed_experts: experts that hand their input on, and a shared expert, need a block "
                             "arrangement that adds the routed rows up itself")
         n, top, width = self.rows.shape
@@ -56,6 +61,8 @@ class RoutedExperts(FeedForward):
         if spec.shared is not None:
             for local, ts in part_class("ffn", spec.shared).tensors(spec.shared).items():
                 t["shared." + local] = ts
+            if spec.shared_gate:
+                t["shared.sg"] = TensorSpec((1, spec.hidden))
         for e in range(spec.experts):
             t[f"e{e}.gate"] = TensorSpec((spec.intermediate, spec.hidden))
             t[f"e{e}.up"] = TensorSpec((spec.intermediate, spec.hidden))
@@ -73,12 +80,20 @@ class RoutedExperts(FeedForward):
         self.spec = spec
         # the router's logits are 32-bit sums whatever its matrix is stored in (`ops.route`)
         self.router = to_compute(tensors["router"], dtype, device)
+        if spec.shared_gate and (spec.shared is None or spec.identity):
+            raise SpecError("routed_experts: a gate on the shared expert needs a shared expert, and a router whose outputs "
+                            "are all experts")
+        if spec.weight_on_input and spec.identity:
+            raise SpecError("routed_experts: weights on the experts' inputs do not go with outputs that hand the input on")
+        if spec.shared_gate:                         # (the gate's row behind the router's: one walk over h serves both)
+            self.router = torch.cat([self.router, to_compute(tensors["shared.sg"], dtype, device).view(1, -1)], dim=0).contiguous()
         self.correction = (tensors["correction"].to(device=device, dtype=torch.float32).contiguous()
                            if spec.correction else None)
         self.shared = None
         if spec.shared is not None:
             self.shared = part_class("ffn", spec.shared)(
-                spec.shared, {k[len("shared."):]: v for k, v in tensors.items() if k.startswith("shared.")}, dtype, device)
+                spec.shared, {k[len("shared."):]: v for k, v in tensors.items() if k.startswith("shared.") and k != "shared.sg"},
+                dtype, device)
         E = spec.experts
         gate_up = torch.stack([torch.cat([to_compute(tensors[f"e{e}.gate"], dtype, device),
                                           to_compute(tensors[f"e{e}.up"], dtype, device)], dim=0) for e in range(E)])
@@ -92,13 +107,22 @@ class RoutedExperts(FeedForward):
 
     def forward(self, ctx, h):
         s = self.spec
-        sel, weights = ops.route(h, self.router, s.top, s.scale, s.score, s.renormalize, self.correction)
+        if hasattr(h, "materialize"):
+            h = h.materialize()
+        gate = None
+        if s.shared_gate:
+            sel, weights, gate = ops.route(h, self.router, s.top, s.scale, s.score, s.renormalize, self.correction, gates=1)
+        else:
+            sel, weights = ops.route(h, self.router, s.top, s.scale, s.score, s.renormalize, self.correction)
         rows = ops.experts_forward(h, sel, self.gate_up, self.down, s.limit, s.alpha,
-                                   ff=s.intermediate if self.tiled else None)
+                                   ff=s.intermediate if self.tiled else None,
+                                   in_weight=weights if s.weight_on_input else None)
         extra = self.shared.forward(ctx, h) if self.shared is not None else None
-        if s.identity == 0 and extra is None:
+        if s.weight_on_input:
+            weights = None
+        if s.identity == 0 and extra is None and weights is not None:
             return RoutedRows(rows, weights)
-        return RoutedRows(rows, weights, sel if s.identity else None, s.experts, extra)
+        return RoutedRows(rows, weights, sel if s.identity else None, s.experts, extra, gate)
 
 
 @register_ffn("clamped_mlp")

@@ -20,13 +20,20 @@ class TableEmbedding(Embedding):
 
     @classmethod
     def tensors(cls, spec) -> Dict[str, TensorSpec]:
-        return {spec.name: TensorSpec((spec.vocab_size, spec.hidden), "matrix")}
+        t = {spec.name: TensorSpec((spec.vocab_size, spec.hidden), "matrix")}
+        if getattr(spec, "side_name", None):
+            t[spec.side_name] = TensorSpec((spec.vocab_size, spec.side_width), "matrix")
+        return t
 
     def __init__(self, spec, tensors: Dict[str, torch.Tensor], dtype, device):
         self.spec = spec
         self.table = to_compute(tensors[spec.name], dtype, device)
+        # a second table whose rows for the step's tokens the layers take slices of (`ctx.side_rows`)
+        self.side_table = to_compute(tensors[spec.side_name], dtype, device) if getattr(spec, "side_name", None) else None
 
     def forward(self, ctx) -> torch.Tensor:
+        if self.side_table is not None:
+            ctx.side_rows = ops.embed_gather(self.side_table, ctx.token_ids)
         scale, wide = float(getattr(self.spec, "scale", 1.0)), bool(getattr(self.spec, "wide", False))
         if wide:
             # 32-bit rows for a stream that is kept so: the factor meets the table's values unrounded

@@ -10,6 +10,11 @@ attention runs over the cached rows [c | k_rot] with ONE key/value head whose va
 which is the shape that the paged attention kernels of this package take (a group of `heads` query heads on one
 key/value head).  Behind it W_uv,h turns a head's mixed latent row into its value.  The cache holds the row twice, as
 the kernels want their operands: as a row among the keys and as a column among the values.
+
+Options of the spec: the queries through a low-rank row of their own (`q_rank`: q = W_uq rmsnorm(W_dq h) * w, two
+products and a norm in place of one product), neighbours paired in the turn (the position's `pairing`), a window, a
+learned term a head in the softmax's denominator (`sink`: the attention kernels take one value a query head), and one gate
+value a head (`gate_per_head`).
 """
 from __future__ import annotations
 
@@ -31,16 +36,21 @@ class LatentAttention(Mixer):
     @classmethod
     def tensors(cls, spec: LatentAttentionSpec) -> Dict[str, TensorSpec]:
         H, d, r, dv, rank = spec.n_heads, spec.head_dim, spec.rot_dim, spec.v_dim, spec.kv_rank
-        t = {
-            "q": TensorSpec((H * (d + r), spec.hidden)),
+        t = {"q": TensorSpec((H * (d + r), spec.hidden))}
+        if spec.q_rank:
+            t = {"dq": TensorSpec((spec.q_rank, spec.hidden)), "dq.norm": TensorSpec((spec.q_rank,), "norm"),
+                 "uq": TensorSpec((H * (d + r), spec.q_rank))}
+        t.update({
             "dkv": TensorSpec((rank + r, spec.hidden)),
             "dkv.norm": TensorSpec((rank,), "norm"),
             "uk": TensorSpec((H * d, rank)),
             "uv": TensorSpec((H * dv, rank)),
             "o": TensorSpec((spec.hidden, H * dv)),
-        }
+        })
+        if spec.sink:
+            t["sink"] = TensorSpec((H,))
         if spec.gate:
-            t["g"] = TensorSpec((H * dv, spec.hidden))
+            t["g"] = TensorSpec((H * (1 if spec.gate_per_head else dv), spec.hidden))
         return t
 
     @classmethod
@@ -53,12 +63,20 @@ class LatentAttention(Mixer):
             raise SpecError(f"latent_attention: kv_rank + rot_dim = {D} is outside 1..512, the range of the attention kernels")
         self.spec = spec
         self.position = part_class("position", spec.position)(spec.position, {}, dtype, device)
-        if self.position.rot_dim > spec.rot_dim or self.position.interleaved:
-            raise SpecError("latent_attention: the rotation turns halves of at most rot_dim features")
+        if self.position.rot_dim > spec.rot_dim:
+            raise SpecError("latent_attention: the rotation turns at most rot_dim features")
         H, d, dv, rank = spec.n_heads, spec.head_dim, spec.v_dim, spec.kv_rank
-        stacked = [tensors["q"], tensors["dkv"]] + ([tensors["g"]] if spec.gate else [])
-        self.proj = Linear(stacked, dtype, device)
-        self.q_off, self.down_off, self.g_off = 0, H * (d + spec.rot_dim), H * (d + spec.rot_dim) + D
+        own_q = [] if spec.q_rank else [tensors["q"]]
+        self.proj = Linear(own_q + [tensors["dkv"]] + ([tensors["g"]] if spec.gate else []), dtype, device)
+        self.q_off = 0
+        self.down_off = 0 if spec.q_rank else H * (d + spec.rot_dim)
+        self.g_off = self.down_off + D
+        self.q_down = self.q_up = self.q_norm_w = None
+        if spec.q_rank:
+            self.q_down = Linear([tensors["dq"]], dtype, device)
+            self.q_up = Linear([tensors["uq"]], dtype, device)
+            self.q_norm_w = tensors["dq.norm"].to(device=device, dtype=torch.float32).contiguous()
+        self.sinks = tensors["sink"].to(device=device, dtype=torch.float32).contiguous() if spec.sink else None
         self.norm_w = tensors["dkv.norm"].to(device=device, dtype=torch.float32).contiguous()
         # W_uk,h^T as [H, rank, d]: the query side of the keys' up-projection; W_uv,h as [H, dv, rank]
         self.uk_t = to_compute(tensors["uk"], dtype, device).view(H, d, rank).transpose(1, 2).contiguous()
@@ -71,17 +89,21 @@ class LatentAttention(Mixer):
         D = rank + r
         group = ctx.groups[cache.group]
         proj = self.proj(h)                                      # [n, q | down, k_rot | g]
+        q_rows = None                                            # the queries' rows where a product of their own made them
+        if self.q_down is not None:
+            q_rows = self.q_up(ops.rmsnorm(self.q_down(h), self.q_norm_w, s.norm_eps))
         table = ctx.position_table(self.position)
         cos, sin = table if table is not None else (None, None)
-        q = ops.latent_prep(proj, heads=H, dim=d, rot_dim=r, rank=rank, rotated=self.position.rot_dim if cos is not None else 0,
+        q = ops.latent_prep(proj, interleaved=self.position.interleaved, q_rows=q_rows, heads=H, dim=d, rot_dim=r, rank=rank, rotated=self.position.rot_dim if cos is not None else 0,
                             q_off=self.q_off, down_off=self.down_off, norm_weight=self.norm_w, eps=s.norm_eps,
                             cos=cos, sin=sin, magnitude=self.position.magnitude, k_cache=cache.k, v_cache=cache.v,
                             slots=group.slots if cache.writable else None, page_size=group.page_size)
         n = q.shape[0]
         # the plain query parts through W_uk^T, into the first `rank` features of every head's query
-        ops.head_product(proj, self.uk_t, x_off=self.q_off, x_head=d + r, out=q.view(n, H * D), o_head=D)
+        ops.head_product(proj if q_rows is None else q_rows, self.uk_t, x_off=self.q_off, x_head=d + r,
+                         out=q.view(n, H * D), o_head=D)
         if ops.attention_mfma_fits(q.dtype, D, group.page_size):
-            common = dict(window=s.window, scale=s.scale)
+            common = dict(window=s.window, scale=s.scale, sinks=self.sinks)
             if 0 < ctx.n_single < ctx.n_seqs:
                 a = ops.attention_mfma(q, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table,
                                        max_q_len=1, max_kv_len=ctx.max_kv_single, seqs=(0, ctx.n_single),
@@ -95,8 +117,8 @@ class LatentAttention(Mixer):
                                        max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len, **common)
         else:
             a = ops.attention_generic(q, cache.k, cache.v, ctx.positions, ctx.token_seq, group.block_table,
-                                      window=s.window, scale=s.scale, max_kv_len=ctx.max_kv_len)
+                                      window=s.window, scale=s.scale, max_kv_len=ctx.max_kv_len, sinks=self.sinks)
         # a [n, H, D]: its first `rank` features are the mixed latent rows; through W_uv, times the gate
         joined = ops.head_product(a.view(n, H * D), self.uv, x_head=D,
-                                  gate=proj if s.gate else None, g_off=self.g_off)
+                                  gate=proj if s.gate else None, g_off=self.g_off, gate_per_head=s.gate_per_head)
         return self.o(joined)

@@ -55,9 +55,24 @@ def yarn_scaling(inv_freq: np.ndarray, factor: float, original: float, fast: flo
     return (f / factor * ramp + f * (1.0 - ramp)).astype(np.float32), 0.1 * math.log(factor) + 1.0
 
 
+def llama3_scaling(inv_freq: np.ndarray, factor: float, low: float, high: float, original: float) -> np.ndarray:
+    """By wavelength l = 2 pi / f: f stays where l < original / high, becomes f / factor where l > original / low, and
+    between the two, with s = (original / l - low) / (high - low), (1 - s) f / factor + s f.  (The frequency scaling of
+    Llama 3.1; Grattafiori et al., "The Llama 3 Herd of Models".)"""
+    if not (factor > 0.0 and original > 0.0 and high > low >= 0.0):
+        raise SpecError(f"rotary scaling 'llama3' needs factor > 0, original > 0 and high > low, got factor={factor} "
+                        f"low={low} high={high} original={original}")
+    f = inv_freq.astype(np.float64)
+    wave = 2.0 * math.pi / f
+    s = (original / wave - low) / (high - low)
+    blended = (1.0 - s) * f / factor + s * f
+    out = np.where(wave < original / high, f, np.where(wave > original / low, f / factor, blended))
+    return out.astype(np.float32)
+
+
 # name of a scaling law -> (inverse frequencies, the law's numbers) -> inverse frequencies, or (inverse frequencies,
 # factor on cos and sin); a law that needs the base and the rotated size says so in SCALING_NEEDS_GEOMETRY
-SCALING_LAWS = {"linear": linear_scaling, "yarn": yarn_scaling}
+SCALING_LAWS = {"linear": linear_scaling, "yarn": yarn_scaling, "llama3": llama3_scaling}
 SCALING_NEEDS_GEOMETRY = {"yarn"}
 
 
