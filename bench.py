@@ -18,13 +18,15 @@ choice): `mixed16` is 16 requests with prompts of 128 to 4,096 random tokens in 
 `--decode-tokens` tokens.  Its JSON line gives tokens a second over the whole run, the prompts' and the
 decoded tokens' rates apart, and the time to a request's first token.
 
-    python bench.py --design buketar|lofudra|fisanex [--design-shapes 1k,2k,4k]
+    python bench.py --design buketar|lofudra|fisanex|ligizen [--design-shapes 1k,2k,4k]
 
 measures the Buketar design (latent attention, gated recurrences, routed experts, residual streams), the Lofudra
 design (windowed sink attention beside retention, matrix memory, state space, norms on both sides) or the Fisanex design
 (a stream normed after every sum, gated window attention with values narrower than keys over caches that layers share,
 routed experts with outputs that hand the input on and a shared expert) at a few layer
-sizes beside the dense decoder at equal width, layers and feed-forward products a token: prompts of `--prefill-tokens`
+sizes beside the dense decoder at equal width, layers and feed-forward products a token, or the Ligizen design (one layer
+norm a layer that both sub-layers read, latent window attention with learned sinks beside chunked attention over caches
+that layers share, experts weighted on their inputs, a token's own input a layer) beside the Fisanex design at equal size: prompts of `--prefill-tokens`
 tokens, decode steps at `--batch` and at batch 1 through the serving loop, and every kernel's time in one prompt and one
 decode step of both.  One JSON line; the default record above is not touched by it.
 
@@ -461,6 +463,43 @@ FISANEX_LIKE_KERNEL = {"postnorm_step": "add_rmsnorm", "qk_rope_kv_strided": "qk
                        "route_plan": "rmsnorm", "attention_mfma": "attention_mfma"}
 
 
+# ---- the Ligizen design beside the Fisanex design at equal size (`--design ligizen`) ---------------------------
+# Layer sizes in the range of real models of its kind.  Even layers: latent attention with a cached row of 256 (latent 192 +
+# 64 turned, neighbours paired), heads of 64 + 64 with values of 64, queries through a row of width / 2, a window of 1,024,
+# learned sinks, and a gated feed-forward of 3 x width.  Odd layers: attention with keys and values of 128 over a quarter as
+# many key heads in chunks of 1,024, half of a head turning with stretched frequencies, every second of them reading the
+# keys and values of the one before it, and routed experts (32, 4 a token, a shared expert of twice their size behind its
+# gate).  A token's own input of 256 in every layer.  The twin is the Fisanex design at the same width and layers (its
+# closest relative in this package: gated attention over shared caches, the same experts and shared expert).
+def ligizen_shape(width: int, layers: int, vocab: int = 32768):
+    heads = width // 128
+    lat = {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": 64, "q_rank": width // 2, "kv_rank": 192, "scale": 128 ** -0.5,
+           "mask": {"size": 1024}, "rot": {"base": 10000.0, "dims": 64}}
+    att = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 0.09, "mask": {"size": 1024},
+           "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    ff = 3 * width // 4 // 64 * 64
+    moe = {"kind": "moe", "router": {"experts": 32, "top": 4}, "expert": {"ff": ff, "limit": 7.0}, "shared": {"ff": 2 * ff, "limit": 7.0}}
+    out = []
+    for i in range(layers):
+        if i % 2 == 0:
+            out.append({"type": "latent_attention", "mixer": dict(lat), "mlp": {"kind": "dense", "ff": 3 * width}})
+        else:
+            out.append({"type": "attention", "mixer": dict(att, kv_from=i - 2) if i % 4 == 3 else dict(att), "mlp": moe})
+    return {"architecture": "Ligizen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
+            "logit_softcap": 30.0, "token_side": {"dim": 256}, "layers": out}
+
+
+def ligizen_twin(b: dict, vocab: int = 32768) -> dict:
+    return fisanex_shape(b["width"], b["layers"], vocab)
+
+
+LIGIZEN_LIKE_KERNEL = {"parallel_step": "postnorm_step", "qk_rope_kv_strided": "qk_rope_kv_strided", "sigmoid_gate": "sigmoid_gate",
+                       "latent_prep": "qk_rope_kv_strided", "head_product": "vendor_gemm", "gate_rows": "clamped_gate_mul",
+                       "experts_gate_up": "experts_gate_up", "experts_down": "experts_down", "route": "route",
+                       "route_plan": "route_plan", "attention_mfma": "attention_mfma", "rmsnorm": "postnorm_step",
+                       "softcap": "scale", "embed_gather": "embed_gather_scaled"}
+
+
 def design_main(args) -> int:
     """Prefill and decode throughput of a design at a few layer sizes beside the dense decoder at equal
     size (random weights), and the time of every kernel of one prefill and one decode step of both."""
@@ -472,7 +511,13 @@ def design_main(args) -> int:
     from inferrs_amd.engine import Engine
     batch, context, prompt = args.batch, min(args.context, 2048), args.prefill_tokens
     records = {}
-    if args.design == "fisanex":
+    twin_label, twin_cls, twin_vocab = "dense", Qwen3Config, "vocab_size"
+    if args.design == "ligizen":
+        from inferrs_amd.config.ligizen import LigizenConfig
+        shapes, shape_of, twin_of, config_cls, like = FISANEX_SHAPES, ligizen_shape, ligizen_twin, LigizenConfig, LIGIZEN_LIKE_KERNEL
+        title, beside = "Ligizen", "Fisanex at equal width and layers"
+        twin_label, twin_cls, twin_vocab = "fisanex", FisanexConfig, "vocab"
+    elif args.design == "fisanex":
         shapes, shape_of, twin_of, config_cls, like = FISANEX_SHAPES, fisanex_shape, fisanex_twin, FisanexConfig, FISANEX_LIKE_KERNEL
         title, beside = "Fisanex", "Qwen3 dense at equal width and layers, heads of 128 and a feed-forward of 3 x width"
     elif args.design == "lofudra":
@@ -486,7 +531,7 @@ def design_main(args) -> int:
         raw_new, raw_old = shape_of(**b), twin_of(b)
         rec = {}
         for label, config, vocab in ((args.design, config_cls.from_dict(raw_new), raw_new["vocab"]),
-                                     ("dense", Qwen3Config.from_dict(raw_old), raw_old["vocab_size"])):
+                                     (twin_label, twin_cls.from_dict(raw_old), raw_old[twin_vocab])):
             pages = batch * (-(-context // PAGE) + 1) + -(-prompt // PAGE) + 8
             note(f"{name} {label}: random weights, {pages} pages")
             engine = Engine.from_random(config, seed=0, dtype=args.dtype, page_size=PAGE, num_pages=pages, max_seqs=batch + 1)
@@ -542,9 +587,9 @@ def main() -> int:
                     help="workloads: cut prompt portions so that a step's tokens are a multiple of this (0: off)")
     ap.add_argument("--decode-run", type=int, default=8,
                     help="decode steps that the serving loop queues on the GPU at once (1: one at a time)")
-    ap.add_argument("--design", default=None, choices=["buketar", "lofudra", "fisanex"],
+    ap.add_argument("--design", default=None, choices=["buketar", "lofudra", "fisanex", "ligizen"],
                     help="instead of the headline: prefill and decode throughput of this design at a few layer sizes "
-                         "beside the dense decoder at equal size, with every kernel's time")
+                         "beside the dense decoder (ligizen: beside the Fisanex design) at equal size, with every kernel's time")
     ap.add_argument("--design-shapes", default=None, help="with --design: the sizes to run, with commas (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
