@@ -160,6 +160,9 @@ int ia_latent_prep(void* q_out, void* k_cache, void* v_cache, const void* proj, 
                    const float* cos_t, const float* sin_t, const int* slots, int n, int H, int d, int r,
                    int rank, int rd, int q_off, int down_off, int ld_proj, int page_size, float eps,
                    float mag, int interleaved, const void* qrows, int ld_q, int dtype, hipStream_t stream);
+// out[t][j] = x[t][x_off + j] / sqrt(mean_j x[t][x_off + j]^2 + eps) * w[j], j < cols: the RMS norm of a slice of rows of pitch x_ld
+int ia_norm_slice(void* out, const void* x, long long x_ld, int x_off, const float* w, float eps, int rows, int cols,
+                  int dtype, hipStream_t stream);
 // out[t][h][j] = sum_i w[h][j][i] x[t][h][i], optionally times sigmoid(gate[t][h][j]), or, with g_per_head, sigmoid(gate[t][h])
 int ia_head_product(void* out, const void* x, const void* w, const void* gate, int n, int H, int n_out,
                     int k_in, long long x_ld, int x_off, int x_head, long long o_ld, int o_off, int o_head,

@@ -229,12 +229,12 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(T* __restrict__ ac
     for (int a = 0; a < 2; ++a) {
         const int i = 2 * ty + a;
         if (i >= rows) continue;
+        // (in_weight: the pair's weight is a factor on the expert's INPUT, hence on both sums ahead of the limits)
+        const float wi = in_weight != nullptr ? in_weight[order[first + i]] : 1.0f;
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             const int j = col0 + 4 * tx + b;
             if (j >= ff) continue;
-            // (in_weight: the pair's weight is a factor on the expert's INPUT, hence on both sums ahead of the limits)
-            const float wi = in_weight != nullptr ? in_weight[order[first + i]] : 1.0f;
             const float gv = fminf(g[a][b] * wi, limit), uv = fminf(fmaxf(u[a][b] * wi, -limit), limit);
             st(act + (long long)(first + i) * ff + j, gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
         }
@@ -297,6 +297,7 @@ __global__ __launch_bounds__(256) void experts_gate_up_mfma_kernel(bf16_t* __res
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         const int i = 16 * rt + (lane & 15);
+        const float wi = in_weight != nullptr && i < rows ? in_weight[order[first + i]] : 1.0f;
 #pragma unroll
         for (int ft = 0; ft < FT; ++ft) {
             const int j0 = col0 + 16 * (wave * FT + ft) + 4 * (lane >> 4);
@@ -305,7 +306,6 @@ __global__ __launch_bounds__(256) void experts_gate_up_mfma_kernel(bf16_t* __res
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 if (i >= rows || j0 + q >= ff) continue;
-                const float wi = in_weight != nullptr ? in_weight[order[first + i]] : 1.0f;
                 const float gv = fminf(gs[q] * wi, limit), uv = fminf(fmaxf(us[q] * wi, -limit), limit);
                 st(act + (long long)(first + i) * ff + j0 + q, gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
             }

@@ -107,6 +107,34 @@ extern "C" int ia_latent_prep(void* q_out, void* k_cache, void* v_cache, const v
     return 0;
 }
 
+// ---- the RMS norm of a slice of wider rows: out[t][j] = x[t][x_off + j] / sqrt(mean_j x^2 + eps) * w[j] -----------------------------
+// (a low-rank row that shares one product with its neighbours, normed on its way to the product that reads it)
+template <typename T>
+__global__ __launch_bounds__(256) void norm_slice_kernel(T* __restrict__ out, const T* __restrict__ x, long long x_ld, int x_off,
+                                                         const float* __restrict__ w, float eps, int cols) {
+    __shared__ float scratch[16];
+    const T* row = x + (long long)blockIdx.x * x_ld + x_off;
+    float sq = 0.f;
+    for (int j = threadIdx.x; j < cols; j += blockDim.x) {
+        const float v = ld(row + j);
+        sq = fmaf(v, v, sq);
+    }
+    const float rs = 1.0f / sqrtf(block_sum(sq, scratch) / (float)cols + eps);
+    for (int j = threadIdx.x; j < cols; j += blockDim.x) st(out + (long long)blockIdx.x * cols + j, ld(row + j) * rs * w[j]);
+}
+
+extern "C" int ia_norm_slice(void* out, const void* x, long long x_ld, int x_off, const float* w, float eps, int rows, int cols,
+                             int dtype, hipStream_t stream) {
+    IA_CHECK(rows >= 0 && cols > 0 && x_off >= 0 && x_off + cols <= x_ld && w != nullptr, "norm_slice: rows=%d cols=%d at %d of %lld",
+             rows, cols, x_off, x_ld);
+    if (rows == 0) return 0;
+    if (dtype == IA_F32) norm_slice_kernel<float><<<rows, 256, 0, stream>>>((float*)out, (const float*)x, x_ld, x_off, w, eps, cols);
+    else if (dtype == IA_BF16) norm_slice_kernel<bf16_t><<<rows, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, x_ld, x_off, w, eps, cols);
+    else IA_CHECK(false, "norm_slice: unknown dtype %d", dtype);
+    IA_LAUNCH_CHECK("norm_slice");
+    return 0;
+}
+
 // ---- a product with a matrix of its own for every head -------------------------------------------------------------
 // out[t][h][j] = sum_i w[h][j][i] * x[t][h][i]   (j < n_out, i < k_in; w is [H, n_out, k_in])
 // x[t][h] starts at x + t * x_ld + x_off + h * x_head, out[t][h] at out + t * o_ld + o_off + h * o_head.  `gate`

@@ -281,6 +281,24 @@ __global__ void sigmoid_gate_bf16_vec_kernel(bf16_t* __restrict__ a, const bf16_
     }
 }
 
+// The same where `group` columns (a multiple of 8) share one gate value: eight values a thread and one sigmoid
+__global__ void sigmoid_gate_group_bf16_vec_kernel(bf16_t* __restrict__ a, const bf16_t* __restrict__ g, int cols, int g_ld,
+                                                   int g_off, int group, size_t total_vecs) {
+    const int vecs_per_row = cols / 8;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total_vecs; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t row = i / vecs_per_row;
+        const int c = (int)(i - row * vecs_per_row) * 8;
+        const uint4 ar = *(const uint4*)(a + row * cols + c);
+        const float s = 1.0f / (1.0f + expf(-ld(g + row * g_ld + g_off + c / group)));
+        const uint32_t aw[4] = {ar.x, ar.y, ar.z, ar.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            o[j] = pack_bf16x2(__uint_as_float(aw[j] << 16) * s, __uint_as_float(aw[j] & 0xffff0000u) * s);
+        *(uint4*)(a + row * cols + c) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
 // group: columns that share one gate value (1: a value a column; a head's width: a value a head)
 extern "C" int ia_sigmoid_gate(void* a, const void* g, int rows, int cols, int g_ld, int g_off, int group, int dtype,
                                hipStream_t stream) {
@@ -294,6 +312,14 @@ extern "C" int ia_sigmoid_gate(void* a, const void* g, int rows, int cols, int g
         const size_t want = (vecs + block - 1) / block;
         sigmoid_gate_bf16_vec_kernel<<<(unsigned)(want < 65535 * 8 ? want : 65535 * 8), block, 0, stream>>>(
             (bf16_t*)a, (const bf16_t*)g, cols, g_ld, g_off, vecs);
+        IA_LAUNCH_CHECK("sigmoid_gate");
+        return 0;
+    }
+    if (group % 8 == 0 && dtype == IA_BF16 && (((uintptr_t)a) & 15) == 0) {
+        const size_t vecs = total / 8;
+        const size_t want = (vecs + block - 1) / block;
+        sigmoid_gate_group_bf16_vec_kernel<<<(unsigned)(want < 65535 * 8 ? want : 65535 * 8), block, 0, stream>>>(
+            (bf16_t*)a, (const bf16_t*)g, cols, g_ld, g_off, group, vecs);
         IA_LAUNCH_CHECK("sigmoid_gate");
         return 0;
     }

@@ -1248,7 +1248,7 @@ def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
 
 # ---- several residual streams, latent attention, gated recurrence, routed experts -----------------
 from .mix import (clamped_gate_mul, conv_step, embed_gather_scaled, experts_forward, gate_rows, head_product,    # noqa: E402
-                  latent_prep, parallel_step, postnorm_step, rglru_scan, route, scale_inplace, sigmoid_gate, softcap,
+                  latent_prep, norm_slice, parallel_step, postnorm_step, rglru_scan, route, scale_inplace, sigmoid_gate, softcap,
                   streams_open, streams_step)
 from .state import (activation, conv_act_step, exp_gates, group_norm_gate, linear_scan, sandwich_step,   # noqa: E402
                     step_gates)

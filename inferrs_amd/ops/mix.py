@@ -126,6 +126,18 @@ def latent_prep(proj: torch.Tensor, *, heads: int, dim: int, rot_dim: int, rank:
     return q
 
 
+def norm_slice(x: torch.Tensor, x_off: int, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """The RMS norm (32-bit statistics) of the columns x_off .. x_off + len(weight) of 2-D rows, as rows of their own."""
+    _dev(x, weight); _f32(weight, "norm weight")
+    cols = weight.numel()
+    if x.dim() != 2 or x.stride(1) != 1 or x_off < 0 or x_off + cols > x.shape[1]:
+        raise KernelError(f"norm_slice: {cols} columns at {x_off} do not fit rows {tuple(x.shape)}")
+    out = torch.empty((x.shape[0], cols), dtype=x.dtype, device=x.device)
+    _check(library().ia_norm_slice(_p(out), _p(x), x.stride(0), x_off, _p(weight), ctypes.c_float(eps), x.shape[0], cols, _dt(x),
+                                   _stream()))
+    return out
+
+
 def head_product(x: torch.Tensor, w: torch.Tensor, *, x_off: int = 0, x_head: Optional[int] = None,
                  out: Optional[torch.Tensor] = None, o_off: int = 0, o_head: Optional[int] = None,
                  out_dtype: Optional[torch.dtype] = None, gate: Optional[torch.Tensor] = None,

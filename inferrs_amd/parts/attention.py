@@ -140,8 +140,13 @@ class Attention(Mixer):
                 biases += [tensors["k_proj.bias"], tensors["v_proj.bias"]]
             self.k_off, self.v_off, at = at, at + G * d, at + G * d + G * dv
         if spec.gate:
-            stacked.append(tensors["g_proj.weight"])
+            g_w = tensors["g_proj.weight"]
             g_rows = H * (1 if spec.gate_per_head else dv)
+            if g_rows % 8:                           # (rows of zeros keep the fused product's pitch a multiple of 16 bytes,
+                pad = 8 - g_rows % 8                 # which the kernels that walk its rows in 16-byte pieces ask for)
+                g_w = torch.cat([g_w, torch.zeros((pad, g_w.shape[1]), dtype=g_w.dtype, device=g_w.device)], dim=0)
+                g_rows += pad
+            stacked.append(g_w)
             if spec.qkv_bias:                        # (the gate has no bias: zeros keep the one fused product)
                 biases.append(torch.zeros((g_rows,), dtype=tensors["q_proj.bias"].dtype))
             self.g_off, at = at, at + g_rows

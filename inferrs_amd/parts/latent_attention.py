@@ -11,8 +11,8 @@ which is the shape that the paged attention kernels of this package take (a grou
 key/value head).  Behind it W_uv,h turns a head's mixed latent row into its value.  The cache holds the row twice, as
 the kernels want their operands: as a row among the keys and as a column among the values.
 
-Options of the spec: the queries through a low-rank row of their own (`q_rank`: q = W_uq rmsnorm(W_dq h) * w, two
-products and a norm in place of one product), neighbours paired in the turn (the position's `pairing`), a window, a
+Options of the spec: the queries through a low-rank row of their own (`q_rank`: q = W_uq rmsnorm(W_dq h) * w; W_dq shares the
+one product of everything that reads h, a norm of that slice and a second product follow), neighbours paired in the turn (the position's `pairing`), a window, a
 learned term a head in the softmax's denominator (`sink`: the attention kernels take one value a query head), and one gate
 value a head (`gate_per_head`).
 """
@@ -66,14 +66,14 @@ class LatentAttention(Mixer):
         if self.position.rot_dim > spec.rot_dim:
             raise SpecError("latent_attention: the rotation turns at most rot_dim features")
         H, d, dv, rank = spec.n_heads, spec.head_dim, spec.v_dim, spec.kv_rank
-        own_q = [] if spec.q_rank else [tensors["q"]]
-        self.proj = Linear(own_q + [tensors["dkv"]] + ([tensors["g"]] if spec.gate else []), dtype, device)
+        # one product for everything that reads h: [q, or the queries' low-rank row | latent row, key part | gate]
+        first = tensors["dq"] if spec.q_rank else tensors["q"]
+        self.proj = Linear([first, tensors["dkv"]] + ([tensors["g"]] if spec.gate else []), dtype, device)
         self.q_off = 0
-        self.down_off = 0 if spec.q_rank else H * (d + spec.rot_dim)
+        self.down_off = first.shape[0]
         self.g_off = self.down_off + D
-        self.q_down = self.q_up = self.q_norm_w = None
+        self.q_up = self.q_norm_w = None
         if spec.q_rank:
-            self.q_down = Linear([tensors["dq"]], dtype, device)
             self.q_up = Linear([tensors["uq"]], dtype, device)
             self.q_norm_w = tensors["dq.norm"].to(device=device, dtype=torch.float32).contiguous()
         self.sinks = tensors["sink"].to(device=device, dtype=torch.float32).contiguous() if spec.sink else None
@@ -88,13 +88,14 @@ class LatentAttention(Mixer):
         H, d, r, dv, rank = s.n_heads, s.head_dim, s.rot_dim, s.v_dim, s.kv_rank
         D = rank + r
         group = ctx.groups[cache.group]
-        proj = self.proj(h)                                      # [n, q | down, k_rot | g]
+        proj = self.proj(h)                                      # [n, q (or its low-rank row) | down, k_rot | g]
         q_rows = None                                            # the queries' rows where a product of their own made them
-        if self.q_down is not None:
-            q_rows = self.q_up(ops.rmsnorm(self.q_down(h), self.q_norm_w, s.norm_eps))
+        if self.q_up is not None:
+            q_rows = self.q_up(ops.norm_slice(proj, 0, self.q_norm_w, s.norm_eps))
         table = ctx.position_table(self.position)
         cos, sin = table if table is not None else (None, None)
-        q = ops.latent_prep(proj, interleaved=self.position.interleaved, q_rows=q_rows, heads=H, dim=d, rot_dim=r, rank=rank, rotated=self.position.rot_dim if cos is not None else 0,
+        q = ops.latent_prep(proj, heads=H, dim=d, rot_dim=r, rank=rank, rotated=self.position.rot_dim if cos is not None else 0,
+                            interleaved=self.position.interleaved, q_rows=q_rows,
                             q_off=self.q_off, down_off=self.down_off, norm_weight=self.norm_w, eps=s.norm_eps,
                             cos=cos, sin=sin, magnitude=self.position.magnitude, k_cache=cache.k, v_cache=cache.v,
                             slots=group.slots if cache.writable else None, page_size=group.page_size)
