@@ -233,5 +233,8 @@ def forward(cfg: dict, w: T, tokens: Sequence[int], dtype=torch.float64, layers_
         if layers_out is not None:
             layers_out.append(x.clone())
     x = layer_norm(x, w["final.norm"], w["final.norm.b"], eps)
+    logits = x @ w["head"].T
+    if cfg.get("logit_softcap") is None:            # (a model without a cap)
+        return logits
     cap = float(cfg["logit_softcap"])
-    return cap * torch.tanh((x @ w["head"].T) / cap)
+    return cap * torch.tanh(logits / cap)
