@@ -127,6 +127,11 @@ def test_small_kernels(dtype):
         gate, rows = (2 * torch.randn(13, cols, generator=g)).to(dtype), torch.randn(13, ld, generator=g).to(dtype)
         got = ops.gate_rows(dev(gate), dev(rows), off, "gelu_tanh")
         np.testing.assert_allclose(got.float().cpu().numpy(), (pl.gelu_tanh(gate.double()) * rows.double()[:, off:off + cols]).numpy(), **tol)
+    # the RMS norm of a slice of wider rows
+    for cols, ld, off in ((16, 40, 0), (10, 33, 7), (1024, 1300, 8)):
+        rows, w = torch.randn(13, ld, generator=g).to(dtype), 1 + 0.2 * torch.randn(cols, generator=g)
+        got = ops.norm_slice(dev(rows), off, dev(w), 1e-5)
+        np.testing.assert_allclose(got.float().cpu().numpy(), pl.rms_norm(rows.double()[:, off:off + cols], w.double(), 1e-5).numpy(), **tol)
     # a product a head with one gate value a head behind it
     H, n_out, k_in = 3, 8, 16
     x, w = torch.randn(9, H * k_in, generator=g).to(dtype), (torch.randn(H, n_out, k_in, generator=g) / 4).to(dtype)
