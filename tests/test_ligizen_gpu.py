@@ -231,8 +231,8 @@ def attention_case(dtype, nq, nkv, d, dv, page, lens, q_lens, window, chunk, see
     return q, kc, vc, positions, token_seq, table
 
 
-SHAPES = [(4, 2, 16, 8), (5, 5, 12, 20), (4, 1, 128, 64), (2, 2, 64, 64), (8, 1, 128, 128), (3, 1, 48, 48), (6, 1, 160, 160)]
-MASKS = [(0, 1), (0, 17), (0, 64), (0, 96), (0, 300), (0, 5000), (24, 0), (200, 0), (50, 64)]
+SHAPES = [(4, 2, 16, 8), (5, 5, 12, 20), (4, 1, 128, 64), (2, 2, 64, 64), (8, 1, 128, 128), (3, 1, 48, 48), (4, 1, 160, 160)]
+MASKS = [(0, 1), (0, 17), (0, 64), (0, 80), (0, 300), (0, 5000), (24, 0), (200, 0), (50, 64)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -280,7 +280,7 @@ def test_attention_in_chunks_with_sinks(nq, nkv, d, dv, window, chunk, dtype):
 # ---- the router with a gate row, the experts with the weight on their input --------------------------------------
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("E,top,W", [(5, 2, 48), (2, 2, 64), (3, 3, 50), (70, 6, 136), (4, 1, 40), (12, 1, 320)])
+@pytest.mark.parametrize("E,top,W", [(5, 2, 48), (2, 2, 64), (3, 3, 50), (70, 6, 136), (4, 1, 40), (10, 1, 384)])
 def test_router_with_a_gate_row(E, top, W, dtype):
     from inferrs_amd import ops
     g = torch.Generator().manual_seed(E * W)
@@ -304,7 +304,7 @@ def test_router_with_a_gate_row(E, top, W, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("E,top,W,ff", [(5, 2, 48, 24), (3, 3, 50, 30), (6, 2, 64, 32), (12, 1, 320, 64)])
+@pytest.mark.parametrize("E,top,W,ff", [(5, 2, 48, 24), (3, 3, 50, 30), (6, 2, 64, 32), (10, 1, 384, 48)])
 def test_experts_with_the_weight_on_their_input(E, top, W, ff, dtype):
     from inferrs_amd import ops
     g = torch.Generator().manual_seed(E + ff)

@@ -37,7 +37,7 @@ def random_attention(rng: random.Random, sharp: float):
     scaling = None
     if turned and rng.random() < 0.6:
         scaling = (rng.choice([2.0, 4.0, 8.0]), rng.choice([0.5, 1.0]), rng.choice([2.0, 4.0]), rng.choice([32, 64, 512]))
-    return attn(kv * rng.choice([1, 2, 4, 6]), kv, dim, vdim, sharp * rng.choice([0.05, 0.125, 0.3]), rng.choice([1, 7, 16, 33, 64, 96, 100, 1000]),
+    return attn(kv * rng.choice([1, 2, 4, 6]), kv, dim, vdim, sharp * rng.choice([0.05, 0.125, 0.3]), rng.choice([1, 7, 16, 33, 64, 80, 100, 1000]),
                 base=rng.choice([100.0, 10000.0, 500000.0]), turned=max(turned, 0), scaling=scaling)
 
 
@@ -46,7 +46,7 @@ def random_latent(rng: random.Random, sharp: float):
     rank = rng.choice([12, 24, 48 - rot_dim, 64 - rot_dim, 128 - rot_dim, 96]) if rng.random() < 0.7 else rng.choice([10, 30, 50])
     return latent(rng.choice([1, 2, 3, 6, 8]), rng.choice([8, 10, 16, 32]), rot_dim, rng.choice([4, 8, 14, 16, 32]),
                   rng.choice([8, 16, 24, 40]), max(rank, 4), sharp * rng.choice([0.08, 0.125, 0.3]),
-                  rng.choice([1, 7, 16, 33, 64, 96, 100, 1000]), base=rng.choice([100.0, 10000.0, 250000.0]))
+                  rng.choice([1, 7, 16, 33, 64, 80, 100, 1000]), base=rng.choice([100.0, 10000.0, 200000.0]))
 
 
 def random_mlp(rng: random.Random, big: bool):
@@ -63,21 +63,21 @@ def random_mlp(rng: random.Random, big: bool):
 
 def random_config(rng: random.Random, sharp: float) -> dict:
     big = rng.random() < 0.35
-    width = rng.choice([128, 256, 320]) if big else rng.choice([24, 33, 40, 50, 64, 72, 96])
+    width = rng.choice([128, 256, 384]) if big else rng.choice([24, 33, 40, 50, 64, 72, 96])
     layers = []
     for i in range(rng.randint(1, 5)):
         owners = [j for j, L in enumerate(layers) if L["type"] == "attention" and L["mixer"].get("kv_from") is None]
         if owners and rng.random() < 0.35:
             j = rng.choice(owners)
             m = {"type": "attention", "mixer": dict(layers[j]["mixer"], kv_from=j, scale=sharp * rng.choice([0.1, 0.2]),
-                                                    mask={"size": rng.choice([1, 5, 24, 64, 96, 300])})}
+                                                    mask={"size": rng.choice([1, 5, 24, 64, 80, 300])})}
             m["mixer"]["heads"] = layers[j]["mixer"]["kv_heads"] * rng.choice([1, 2, 3])
         else:
             m = random_attention(rng, sharp) if rng.random() < 0.5 else random_latent(rng, sharp)
         layers.append(layer(m, random_mlp(rng, big)))
     return model(rng.choice([31, 64, 100, 257, 576]), width, layers, eps=rng.choice([1e-6, 1e-5]),
-                 embed_scale=rng.choice([1.0, 3.0, 17.0]), cap=rng.choice([None, 5.0, 15.0, 30.0]),
-                 side=rng.choice([None, 4, 6, 24]))
+                 embed_scale=rng.choice([1.0, 3.0, 17.0]), cap=rng.choice([None, 5.0, 12.0, 30.0]),
+                 side=rng.choice([None, 4, 6, 20]))
 
 
 def run(folder, cfg, dtype, trace, out_dir):
